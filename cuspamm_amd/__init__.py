@@ -1,0 +1,18 @@
+"""cuspamm_amd -- gfx950 (MI355X) SpAMM engine behind a C ABI.
+
+The compute lives in ``libspamm_gfx950.so`` (hand-written HIP kernels, see
+``csrc/``); this package is the thin host-side mirror of the C ABI declared in
+``include/spamm.h``.  There is no CPU fallback: loading fails loudly when the
+library has not been built (``python -m cuspamm_amd.build``).
+"""
+from .api import (  # noqa: F401
+    ROLE_A,
+    ROLE_B,
+    FLAG_TIMING,
+    SpammContext,
+    SpammError,
+    SpammParams,
+    SpammStats,
+    load_library,
+    library_path,
+)

@@ -1,0 +1,251 @@
+"""ctypes mirror of include/spamm.h.
+
+Matrices are torch CUDA tensors (torch is only the device allocator and stream
+provider); every call goes through the C ABI with raw device pointers.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_NAME = "libspamm_gfx950.so"
+
+ROLE_A = 0
+ROLE_B = 1
+FLAG_A_EQ_B = 1
+FLAG_TIMING = 2
+
+OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV = 0, -1, -2, -3, -4, -5
+
+
+class SpammParams(ctypes.Structure):
+    """spamm_params: run-time form of para.h / main.h constants (M,K,N,LoNum,Norm)."""
+    _fields_ = [("M", ctypes.c_int64), ("K", ctypes.c_int64), ("N", ctypes.c_int64),
+                ("tile", ctypes.c_int32), ("tau", ctypes.c_float),
+                ("flags", ctypes.c_uint32), ("reserved", ctypes.c_uint32)]
+
+
+class SpammStats(ctypes.Structure):
+    _fields_ = [("total_products", ctypes.c_int64), ("kept_products", ctypes.c_int64),
+                ("ms_normmap_a", ctypes.c_float), ("ms_normmap_b", ctypes.c_float),
+                ("ms_gate", ctypes.c_float), ("ms_gemm", ctypes.c_float),
+                ("ms_total", ctypes.c_float), ("timing_valid", ctypes.c_int32)]
+
+
+class SpammError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__("%s failed: %s (code %d)" % (what, _strerror(code), code))
+
+
+_lib = None
+
+
+def library_path():
+    return os.path.join(HERE, _LIB_NAME)
+
+
+def load_library():
+    """Loads libspamm_gfx950.so; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            "%s is missing: build it with `python -m cuspamm_amd.build` "
+            "(the SpAMM engine has no CPU or PyTorch fallback)" % path)
+    # torch ships its own HIP runtime; import it first so that both share one copy.
+    import torch  # noqa: F401
+    L = ctypes.CDLL(path)
+    vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_float
+    L.spamm_create.argtypes = [ctypes.POINTER(vp), ctypes.c_int]
+    L.spamm_destroy.argtypes = [vp]
+    L.spamm_set_stream.argtypes = [vp, vp]
+    L.spamm_multiply.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
+    L.spamm_normmap_f32.argtypes = [vp, ctypes.c_int, vp, i64, i64, i32]
+    L.spamm_gate.argtypes = [vp, f32]
+    L.spamm_gemm_gated.argtypes = [vp, vp]
+    L.spamm_set_normmaps.argtypes = [vp, vp, vp, i64, i64, i64, i32]
+    L.spamm_get_normmap.argtypes = [vp, ctypes.c_int, vp]
+    L.spamm_get_counts.argtypes = [vp, vp]
+    L.spamm_get_klist.argtypes = [vp, vp]
+    L.spamm_get_mask.argtypes = [vp, vp]
+    L.spamm_get_fp16.argtypes = [vp, ctypes.c_int, vp]
+    L.spamm_get_stats.argtypes = [vp, ctypes.POINTER(SpammStats)]
+    L.spamm_fill_decay_f32.argtypes = [vp, vp, i64, i64, vp, ctypes.c_uint64, ctypes.c_int]
+    L.spamm_synchronize.argtypes = [vp]
+    L.spamm_strerror.argtypes = [ctypes.c_int]
+    L.spamm_strerror.restype = ctypes.c_char_p
+    L.spamm_last_hip_error.argtypes = [vp]
+    L.spamm_version.restype = ctypes.c_int
+    _lib = L
+    return L
+
+
+def _strerror(code):
+    try:
+        return load_library().spamm_strerror(code).decode()
+    except Exception:  # pragma: no cover
+        return "?"
+
+
+def _check(code, what):
+    if code != OK:
+        raise SpammError(code, what)
+
+
+def _devptr(t, dtype_name):
+    import torch
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("expected a CUDA tensor")
+    if str(t.dtype) != "torch." + dtype_name:
+        raise TypeError("expected dtype %s, got %s" % (dtype_name, t.dtype))
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous (row-major) tensor")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+class SpammContext:
+    """One device + one stream + reusable workspaces (spamm_ctx)."""
+
+    def __init__(self, device=0, use_torch_stream=True):
+        self._lib = load_library()
+        self._h = ctypes.c_void_p()
+        _check(self._lib.spamm_create(ctypes.byref(self._h), int(device)), "spamm_create")
+        self.device = int(device)
+        self._shape = None
+        if use_torch_stream:
+            import torch
+            self.set_stream(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def close(self):
+        if self._h:
+            self._lib.spamm_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- plumbing
+    def set_stream(self, raw_stream):
+        _check(self._lib.spamm_set_stream(self._h, ctypes.c_void_p(raw_stream or 0)),
+               "spamm_set_stream")
+
+    def synchronize(self):
+        _check(self._lib.spamm_synchronize(self._h), "spamm_synchronize")
+
+    def last_hip_error(self):
+        return int(self._lib.spamm_last_hip_error(self._h))
+
+    # -- the multiply call
+    def multiply(self, A, B, tile, tau, C=None, timing=False):
+        import torch
+        if A.dim() != 2 or B.dim() != 2:
+            raise ValueError("A and B must be matrices")
+        M, K = A.shape
+        K2, N = B.shape
+        if K != K2:
+            raise ValueError("inner dimensions differ")
+        if C is None:
+            C = torch.empty((M, N), dtype=torch.float32, device=A.device)
+        p = SpammParams(M, K, N, int(tile), float(tau), FLAG_TIMING if timing else 0, 0)
+        _check(self._lib.spamm_multiply(self._h, ctypes.byref(p), _devptr(A, "float32"),
+                                        _devptr(B, "float32"), _devptr(C, "float32")),
+               "spamm_multiply")
+        self._shape = (M // tile, K // tile, N // tile, int(tile), M, K, N)
+        return C
+
+    def multiply_raw(self, params, dA, dB, dC):
+        """Pointer-level call (ints are raw device addresses); returns the error code."""
+        return int(self._lib.spamm_multiply(self._h, ctypes.byref(params), ctypes.c_void_p(dA),
+                                            ctypes.c_void_p(dB), ctypes.c_void_p(dC)))
+
+    # -- stages
+    def normmap_f32(self, role, X, tile):
+        rows, cols = X.shape
+        _check(self._lib.spamm_normmap_f32(self._h, int(role), _devptr(X, "float32"), rows, cols,
+                                           int(tile)), "spamm_normmap_f32")
+        s = list(self._shape) if self._shape and self._shape[3] == tile else [0, 0, 0, tile, 0, 0, 0]
+        if role == ROLE_A:
+            s[0], s[1], s[4], s[5] = rows // tile, cols // tile, rows, cols
+        else:
+            s[1], s[2], s[5], s[6] = rows // tile, cols // tile, rows, cols
+        self._shape = tuple(s)
+
+    def set_normmaps(self, nA, nB, tile):
+        nA = np.ascontiguousarray(nA, dtype=np.float32)
+        nB = np.ascontiguousarray(nB, dtype=np.float32)
+        nbM, nbK = nA.shape
+        nbK2, nbN = nB.shape
+        if nbK != nbK2:
+            raise ValueError("norm map shapes differ")
+        _check(self._lib.spamm_set_normmaps(self._h, nA.ctypes.data, nB.ctypes.data, nbM, nbK, nbN,
+                                            int(tile)), "spamm_set_normmaps")
+        self._shape = (nbM, nbK, nbN, int(tile), nbM * tile, nbK * tile, nbN * tile)
+
+    def gate(self, tau):
+        _check(self._lib.spamm_gate(self._h, float(tau)), "spamm_gate")
+
+    def gemm_gated(self, C):
+        _check(self._lib.spamm_gemm_gated(self._h, _devptr(C, "float32")), "spamm_gemm_gated")
+        return C
+
+    # -- read-back
+    def get_normmap(self, role):
+        nbM, nbK, nbN = self._shape[:3]
+        shp = (nbM, nbK) if role == ROLE_A else (nbK, nbN)
+        out = np.empty(shp, dtype=np.float32)
+        _check(self._lib.spamm_get_normmap(self._h, int(role), out.ctypes.data), "spamm_get_normmap")
+        return out
+
+    def get_counts(self):
+        nbM, nbK, nbN = self._shape[:3]
+        out = np.empty((nbM, nbN), dtype=np.int32)
+        _check(self._lib.spamm_get_counts(self._h, out.ctypes.data), "spamm_get_counts")
+        return out
+
+    def get_klist(self):
+        nbM, nbK, nbN = self._shape[:3]
+        out = np.empty((nbM, nbN, nbK), dtype=np.uint16)
+        _check(self._lib.spamm_get_klist(self._h, out.ctypes.data), "spamm_get_klist")
+        return out
+
+    def get_mask(self):
+        nbM, nbK, nbN = self._shape[:3]
+        out = np.empty((nbM, nbN, (nbK + 63) // 64), dtype=np.uint64)
+        _check(self._lib.spamm_get_mask(self._h, out.ctypes.data), "spamm_get_mask")
+        return out
+
+    def get_fp16(self, role):
+        M, K, N = self._shape[4:7]
+        shp = (M, K) if role == ROLE_A else (K, N)
+        out = np.empty(shp, dtype=np.uint16)
+        _check(self._lib.spamm_get_fp16(self._h, int(role), out.ctypes.data), "spamm_get_fp16")
+        return out
+
+    def get_stats(self):
+        st = SpammStats()
+        _check(self._lib.spamm_get_stats(self._h, ctypes.byref(st)), "spamm_get_stats")
+        return st
+
+    # -- synthetic inputs
+    def fill_decay(self, X, table, seed, random=True):
+        rows, cols = X.shape
+        table = np.ascontiguousarray(table, dtype=np.float32)
+        if table.size < max(rows, cols):
+            raise ValueError("decay table shorter than max(rows, cols)")
+        _check(self._lib.spamm_fill_decay_f32(self._h, _devptr(X, "float32"), rows, cols,
+                                              table.ctypes.data, int(seed), 1 if random else 0),
+               "spamm_fill_decay_f32")
+        return X

@@ -1,0 +1,66 @@
+"""Builds libspamm_gfx950.so (HIP kernels + C ABI) in-tree with hipcc.
+
+Usage: ``python -m cuspamm_amd.build`` (or ``build_library()`` from Python).
+The library is cross-compiled for gfx950 and needs no GPU to build.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(HERE, "libspamm_gfx950.so")
+
+SOURCES = ["kernels_normmap.hip", "kernels_gate.hip", "kernels_gemm.hip", "spamm_api.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -packed-fp32-ops is switched off on purpose: the compiler must not form
+# v_pk_{add,mul,fma}_f32 from the norm accumulation.
+CFLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fvisibility=hidden",
+    "-Wall",
+    "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(
+        line for line in proc.stdout.splitlines()
+        if "packed-fp32-ops" not in line or "is not a recognized feature" not in line
+    )
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_library(verbose=False):
+    """Compiles every HIP source and links the shared library. Always rebuilds."""
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        return _run([HIPCC] + CFLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        logs = list(ex.map(compile_one, zip(SOURCES, objs)))
+    logs.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs))
+    if verbose:
+        for text in logs:
+            if text.strip():
+                print(text)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))
+    sys.exit(0)

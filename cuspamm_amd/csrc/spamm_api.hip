@@ -1,0 +1,404 @@
+// C ABI of libspamm_gfx950.so: the host driver that replaces the timed body of
+// the reference's main() (cuSpAMM.cu:458-546) and its per-device plan
+// (TGPUplan, cuSpAMM.cu:6-12, 433-451).  See include/spamm.h for the contract.
+#include "../../include/spamm.h"
+
+#include <new>
+#include <string.h>
+#include <vector>
+
+#include "spamm_internal.h"
+
+using namespace spamm;
+
+namespace {
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+};
+
+}  // namespace
+
+struct spamm_ctx {
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    int last_hip = 0;
+
+    // problem shape of the current workspace contents
+    int64_t M = 0, K = 0, N = 0;
+    int tile = 0;
+    bool have_a = false, have_b = false, have_gate = false;
+    float tau = 0.0f;
+
+    DevBuf packedA, packedB, nA, nB, nBt;
+    DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, kept_total;
+    DevBuf scratch;   // read-back staging / decay table
+
+    hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    bool timing = false;        // events of the last multiply are valid
+    bool ev_a = false, ev_b = false, ev_gate = false, ev_gemm = false;
+};
+
+namespace {
+
+#define HIPCHK(ctx, call)                         \
+    do {                                          \
+        hipError_t e__ = (call);                  \
+        if (e__ != hipSuccess) {                  \
+            (ctx)->last_hip = (int)e__;           \
+            (void)hipGetLastError();              \
+            return e__ == hipErrorOutOfMemory ? SPAMM_ENOMEM : SPAMM_EHIP; \
+        }                                         \
+    } while (0)
+
+int ensure(spamm_ctx *c, DevBuf &b, size_t bytes) {
+    if (bytes == 0) bytes = 16;
+    if (b.cap >= bytes) return SPAMM_OK;
+    if (b.p) {
+        HIPCHK(c, hipStreamSynchronize(c->stream));
+        HIPCHK(c, hipFree(b.p));
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    HIPCHK(c, hipMalloc(&b.p, bytes));
+    b.cap = bytes;
+    return SPAMM_OK;
+}
+
+bool tile_ok(int t) { return t == 32 || t == 64 || t == 128; }
+
+struct Shape {
+    int64_t nbM, nbK, nbN, words, n_macro;
+};
+
+Shape shape_of(const spamm_ctx *c) {
+    Shape s;
+    s.nbM = c->M / c->tile;
+    s.nbK = c->K / c->tile;
+    s.nbN = c->N / c->tile;
+    s.words = (s.nbK + 63) / 64;
+    const int MT = macro_dim(c->tile);
+    s.n_macro = ((s.nbM + MT - 1) / MT) * ((s.nbN + MT - 1) / MT);
+    return s;
+}
+
+GateBuffers gate_buffers(spamm_ctx *c) {
+    GateBuffers g;
+    g.nA = (const float *)c->nA.p;
+    g.nBt = (const float *)c->nBt.p;
+    g.counts = (int32_t *)c->counts.p;
+    g.klist = (uint16_t *)c->klist.p;
+    g.mask = (uint64_t *)c->mask.p;
+    g.macro_list = (MacroEntry *)c->macro_list.p;
+    g.macro_count = (int32_t *)c->macro_count.p;
+    g.macro_work = (int32_t *)c->macro_work.p;
+    g.order = (int32_t *)c->order.p;
+    g.kept_total = (int64_t *)c->kept_total.p;
+    return g;
+}
+
+int set_device(spamm_ctx *c) {
+    HIPCHK(c, hipSetDevice(c->device));
+    return SPAMM_OK;
+}
+
+// Called when an operand with a different shape/tile arrives: everything
+// derived from the old shape is stale.
+void reset_shape(spamm_ctx *c, int tile) {
+    c->tile = tile;
+    c->M = c->K = c->N = 0;
+    c->have_a = c->have_b = c->have_gate = false;
+}
+
+int copy_out(spamm_ctx *c, const void *dev, void *host, size_t bytes) {
+    HIPCHK(c, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return SPAMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int spamm_version(void) { return 100; }
+
+const char *spamm_strerror(int code) {
+    switch (code) {
+        case SPAMM_OK: return "ok";
+        case SPAMM_EINVAL: return "invalid argument (dimension not a multiple of tile, tile not in {32,64,128}, null pointer, or size limit)";
+        case SPAMM_ENOMEM: return "out of memory";
+        case SPAMM_EHIP: return "HIP runtime error (see spamm_last_hip_error)";
+        case SPAMM_ESTATE: return "stage called before the stage it depends on";
+        case SPAMM_ENODEV: return "no usable gfx950 device";
+        default: return "unknown error";
+    }
+}
+
+int spamm_create(spamm_ctx **out, int device) {
+    if (!out) return SPAMM_EINVAL;
+    *out = nullptr;
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0) {
+        (void)hipGetLastError();
+        return SPAMM_ENODEV;
+    }
+    if (device < 0 || device >= ndev) return SPAMM_EINVAL;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return SPAMM_ENODEV;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return SPAMM_ENODEV;
+    spamm_ctx *c = new (std::nothrow) spamm_ctx();
+    if (!c) return SPAMM_ENOMEM;
+    c->device = device;
+    int rc = set_device(c);
+    if (rc != SPAMM_OK) { delete c; return rc; }
+    if (hipStreamCreate(&c->own_stream) != hipSuccess) { delete c; return SPAMM_EHIP; }
+    c->stream = c->own_stream;
+    for (int i = 0; i < 5; i++)
+        if (hipEventCreate(&c->ev[i]) != hipSuccess) { delete c; return SPAMM_EHIP; }
+    if (gemm_init() != hipSuccess) { delete c; return SPAMM_EHIP; }
+    *out = c;
+    return SPAMM_OK;
+}
+
+int spamm_destroy(spamm_ctx *c) {
+    if (!c) return SPAMM_EINVAL;
+    (void)hipSetDevice(c->device);
+    (void)hipStreamSynchronize(c->stream);
+    DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->counts, &c->klist,
+                      &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
+                      &c->kept_total, &c->scratch};
+    for (DevBuf *b : bufs)
+        if (b->p) (void)hipFree(b->p);
+    for (int i = 0; i < 5; i++)
+        if (c->ev[i]) (void)hipEventDestroy(c->ev[i]);
+    if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
+    delete c;
+    return SPAMM_OK;
+}
+
+int spamm_set_stream(spamm_ctx *c, void *hip_stream) {
+    if (!c) return SPAMM_EINVAL;
+    c->stream = hip_stream ? (hipStream_t)hip_stream : c->own_stream;
+    return SPAMM_OK;
+}
+
+int spamm_last_hip_error(spamm_ctx *c) { return c ? c->last_hip : 0; }
+
+int spamm_synchronize(spamm_ctx *c) {
+    if (!c) return SPAMM_EINVAL;
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return SPAMM_OK;
+}
+
+int spamm_normmap_f32(spamm_ctx *c, int role, const float *dX, int64_t rows, int64_t cols,
+                      int32_t tile) {
+    if (!c || !dX || !tile_ok(tile)) return SPAMM_EINVAL;
+    if (role != SPAMM_ROLE_A && role != SPAMM_ROLE_B) return SPAMM_EINVAL;
+    if (rows <= 0 || cols <= 0 || rows % tile || cols % tile) return SPAMM_EINVAL;
+    if (rows / tile > 65535 || cols / tile > 65535) return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    if (c->tile != tile) reset_shape(c, tile);
+    const size_t nt = (size_t)(rows / tile) * (size_t)(cols / tile);
+    if (role == SPAMM_ROLE_A) {
+        // a new A invalidates B only if the shared dimension K changes
+        if (c->have_b && c->K != cols) c->have_b = false;
+        c->M = rows;
+        c->K = cols;
+        if ((rc = ensure(c, c->packedA, (size_t)rows * cols * 2))) return rc;
+        if ((rc = ensure(c, c->nA, nt * 4))) return rc;
+        if (c->timing) HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
+        HIPCHK(c, launch_normmap_a(dX, rows, cols, tile, c->packedA.p, (float *)c->nA.p, c->stream));
+        if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[2], c->stream)); c->ev_a = true; }
+        c->have_a = true;
+    } else {
+        if (c->have_a && c->K != rows) c->have_a = false;
+        c->K = rows;
+        c->N = cols;
+        if ((rc = ensure(c, c->packedB, (size_t)rows * cols * 2))) return rc;
+        if ((rc = ensure(c, c->nB, nt * 4))) return rc;
+        if ((rc = ensure(c, c->nBt, nt * 4))) return rc;
+        if (c->timing) HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
+        HIPCHK(c, launch_normmap_b(dX, rows, cols, tile, c->packedB.p, (float *)c->nB.p,
+                                   (float *)c->nBt.p, c->stream));
+        if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[1], c->stream)); c->ev_b = true; }
+        c->have_b = true;
+    }
+    c->have_gate = false;
+    return SPAMM_OK;
+}
+
+int spamm_set_normmaps(spamm_ctx *c, const float *nA, const float *nB, int64_t nbM, int64_t nbK,
+                       int64_t nbN, int32_t tile) {
+    if (!c || !nA || !nB || !tile_ok(tile)) return SPAMM_EINVAL;
+    if (nbM <= 0 || nbK <= 0 || nbN <= 0 || nbM > 65535 || nbK > 65535 || nbN > 65535)
+        return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    reset_shape(c, tile);
+    c->M = nbM * tile;
+    c->K = nbK * tile;
+    c->N = nbN * tile;
+    if ((rc = ensure(c, c->nA, (size_t)nbM * nbK * 4))) return rc;
+    if ((rc = ensure(c, c->nB, (size_t)nbK * nbN * 4))) return rc;
+    if ((rc = ensure(c, c->nBt, (size_t)nbK * nbN * 4))) return rc;
+    HIPCHK(c, hipMemcpyAsync(c->nA.p, nA, (size_t)nbM * nbK * 4, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, hipMemcpyAsync(c->nB.p, nB, (size_t)nbK * nbN * 4, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, launch_transpose_normmap((const float *)c->nB.p, nbK, nbN, (float *)c->nBt.p, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    // norm maps only: the gate may run, the GEMM may not (no operands)
+    c->have_a = c->have_b = false;
+    c->have_gate = false;
+    return SPAMM_OK;
+}
+
+int spamm_gate(spamm_ctx *c, float tau) {
+    if (!c) return SPAMM_EINVAL;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    if (tau != tau) return SPAMM_EINVAL;   // NaN
+    int rc = set_device(c);
+    if (rc) return rc;
+    const Shape s = shape_of(c);
+    if (gate_lds_bytes(c->tile, s.nbK) > 64 * 1024) return SPAMM_EINVAL;
+    const size_t nt = (size_t)s.nbM * s.nbN;
+    if ((rc = ensure(c, c->counts, nt * 4))) return rc;
+    if ((rc = ensure(c, c->klist, nt * s.nbK * 2))) return rc;
+    if ((rc = ensure(c, c->mask, nt * s.words * 8))) return rc;
+    if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
+    if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 4))) return rc;
+    if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
+    if ((rc = ensure(c, c->order, (size_t)s.n_macro * 4))) return rc;
+    if ((rc = ensure(c, c->kept_total, 8))) return rc;
+    if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
+    HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->stream));
+    if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[3], c->stream)); c->ev_gate = true; }
+    c->tau = tau;
+    c->have_gate = true;
+    return SPAMM_OK;
+}
+
+int spamm_gemm_gated(spamm_ctx *c, float *dC) {
+    if (!c || !dC) return SPAMM_EINVAL;
+    if (!c->have_a || !c->have_b || !c->have_gate) return SPAMM_ESTATE;
+    int rc = set_device(c);
+    if (rc) return rc;
+    if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
+    HIPCHK(c, launch_gemm(c->packedA.p, c->packedB.p, gate_buffers(c), c->M, c->K, c->N, c->tile, dC,
+                          c->stream));
+    if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[4], c->stream)); c->ev_gemm = true; }
+    return SPAMM_OK;
+}
+
+int spamm_multiply(spamm_ctx *c, const spamm_params *p, const float *dA, const float *dB,
+                   float *dC) {
+    if (!c || !p || !dA || !dB || !dC) return SPAMM_EINVAL;
+    if (!tile_ok(p->tile)) return SPAMM_EINVAL;
+    if (p->M <= 0 || p->K <= 0 || p->N <= 0) return SPAMM_EINVAL;
+    if (p->M % p->tile || p->K % p->tile || p->N % p->tile) return SPAMM_EINVAL;
+    if (p->tau != p->tau) return SPAMM_EINVAL;
+    c->timing = (p->flags & SPAMM_FLAG_TIMING) != 0;
+    c->ev_a = c->ev_b = c->ev_gate = c->ev_gemm = false;
+    int rc;
+    // same order as the reference: B's norm map first, then A's (cuSpAMM.cu:478-503)
+    if ((rc = spamm_normmap_f32(c, SPAMM_ROLE_B, dB, p->K, p->N, p->tile))) return rc;
+    if ((rc = spamm_normmap_f32(c, SPAMM_ROLE_A, dA, p->M, p->K, p->tile))) return rc;
+    if ((rc = spamm_gate(c, p->tau))) return rc;
+    if ((rc = spamm_gemm_gated(c, dC))) return rc;
+    return SPAMM_OK;
+}
+
+int spamm_get_stats(spamm_ctx *c, spamm_stats *out) {
+    if (!c || !out) return SPAMM_EINVAL;
+    memset(out, 0, sizeof(*out));
+    if (!c->have_gate) return SPAMM_ESTATE;
+    int rc = set_device(c);
+    if (rc) return rc;
+    const Shape s = shape_of(c);
+    out->total_products = s.nbM * s.nbK * s.nbN;
+    int64_t kept = 0;
+    if ((rc = copy_out(c, c->kept_total.p, &kept, 8))) return rc;
+    out->kept_products = kept;
+    if (c->timing && c->ev_a && c->ev_b && c->ev_gate && c->ev_gemm) {
+        HIPCHK(c, hipEventElapsedTime(&out->ms_normmap_b, c->ev[0], c->ev[1]));
+        HIPCHK(c, hipEventElapsedTime(&out->ms_normmap_a, c->ev[1], c->ev[2]));
+        HIPCHK(c, hipEventElapsedTime(&out->ms_gate, c->ev[2], c->ev[3]));
+        HIPCHK(c, hipEventElapsedTime(&out->ms_gemm, c->ev[3], c->ev[4]));
+        HIPCHK(c, hipEventElapsedTime(&out->ms_total, c->ev[0], c->ev[4]));
+        out->timing_valid = 1;
+    }
+    return SPAMM_OK;
+}
+
+int spamm_get_normmap(spamm_ctx *c, int role, float *host_out) {
+    if (!c || !host_out) return SPAMM_EINVAL;
+    if (!c->tile) return SPAMM_ESTATE;
+    const Shape s = shape_of(c);
+    if (role == SPAMM_ROLE_A) {
+        if (!c->nA.p || !c->M || !c->K) return SPAMM_ESTATE;
+        return copy_out(c, c->nA.p, host_out, (size_t)s.nbM * s.nbK * 4);
+    }
+    if (role == SPAMM_ROLE_B) {
+        if (!c->nB.p || !c->K || !c->N) return SPAMM_ESTATE;
+        return copy_out(c, c->nB.p, host_out, (size_t)s.nbK * s.nbN * 4);
+    }
+    return SPAMM_EINVAL;
+}
+
+int spamm_get_counts(spamm_ctx *c, int32_t *host_out) {
+    if (!c || !host_out) return SPAMM_EINVAL;
+    if (!c->have_gate) return SPAMM_ESTATE;
+    const Shape s = shape_of(c);
+    return copy_out(c, c->counts.p, host_out, (size_t)s.nbM * s.nbN * 4);
+}
+
+int spamm_get_klist(spamm_ctx *c, uint16_t *host_out) {
+    if (!c || !host_out) return SPAMM_EINVAL;
+    if (!c->have_gate) return SPAMM_ESTATE;
+    const Shape s = shape_of(c);
+    return copy_out(c, c->klist.p, host_out, (size_t)s.nbM * s.nbN * s.nbK * 2);
+}
+
+int spamm_get_mask(spamm_ctx *c, uint64_t *host_out) {
+    if (!c || !host_out) return SPAMM_EINVAL;
+    if (!c->have_gate) return SPAMM_ESTATE;
+    const Shape s = shape_of(c);
+    return copy_out(c, c->mask.p, host_out, (size_t)s.nbM * s.nbN * s.words * 8);
+}
+
+int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
+    if (!c || !host_out) return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    int64_t rows, cols;
+    const void *packed;
+    if (role == SPAMM_ROLE_A) {
+        if (!c->have_a) return SPAMM_ESTATE;
+        rows = c->M; cols = c->K; packed = c->packedA.p;
+    } else if (role == SPAMM_ROLE_B) {
+        if (!c->have_b) return SPAMM_ESTATE;
+        rows = c->K; cols = c->N; packed = c->packedB.p;
+    } else {
+        return SPAMM_EINVAL;
+    }
+    const size_t bytes = (size_t)rows * cols * 2;
+    if ((rc = ensure(c, c->scratch, bytes))) return rc;
+    HIPCHK(c, launch_unpack(packed, rows, cols, c->tile, role, (uint16_t *)c->scratch.p, c->stream));
+    return copy_out(c, c->scratch.p, host_out, bytes);
+}
+
+int spamm_fill_decay_f32(spamm_ctx *c, float *dX, int64_t rows, int64_t cols,
+                         const float *host_table, uint64_t seed, int random) {
+    if (!c || !dX || !host_table || rows <= 0 || cols <= 0 || cols % 4) return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    const int64_t n = rows > cols ? rows : cols;
+    if ((rc = ensure(c, c->scratch, (size_t)n * 4))) return rc;
+    HIPCHK(c, hipMemcpyAsync(c->scratch.p, host_table, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, launch_fill_decay(dX, rows, cols, (const float *)c->scratch.p, seed, random, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return SPAMM_OK;
+}
+
+}  // extern "C"

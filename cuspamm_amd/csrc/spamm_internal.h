@@ -1,0 +1,70 @@
+// Internal declarations shared by the translation units of libspamm_gfx950.so.
+// Host-side launchers only; kernels live in the .hip files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace spamm {
+
+// ---------------------------------------------------------------------------
+// Packed fp16 operand layout (private to the library).
+//
+// An operand is cut into b x b tiles; every tile is one contiguous block of
+// b*b halves.  Inside a tile the element with free index r (row of A / column
+// of B) and contraction index k (column of A / row of B) sits at
+//     ((k / 8) * b + r) * 8 + (k % 8)          [units: halves]
+// i.e. [k-group][r][8]: a 16-byte vector holds 8 consecutive k of one r, which
+// is exactly one lane's share of an MFMA 32x32x16 operand, and 32 consecutive
+// r are 512 contiguous bytes.  Tile order: A tile (I,Kt) at I*nbK + Kt,
+// B tile (Kt,J) at J*nbK + Kt, so that the k tiles of one output tile are
+// consecutive in memory for both operands.
+// ---------------------------------------------------------------------------
+
+// Output tiles are grouped into macro tiles of (256/b) x (256/b) tiles
+// (256 x 256 elements); one workgroup of the gated GEMM owns one macro tile.
+inline int macro_dim(int tile) { return 256 / tile; }
+
+// One entry of a macro tile's union k list: tile column/row k of the
+// operands plus the set of output tiles (bit a*MT+b = tile row a, column b of
+// the macro tile) that keep the product with this k.  16 bytes so that the
+// GEMM fetches an entry with one scalar load.
+struct __attribute__((aligned(16))) MacroEntry {
+    uint32_t k;
+    uint32_t need;      // bits 0..7: tile rows with any kept product, bits 8..15: tile columns
+    uint32_t mask_lo;
+    uint32_t mask_hi;
+};
+
+struct GateBuffers {
+    const float *nA;        // [nbM x nbK]
+    const float *nBt;       // [nbN x nbK]  (transposed B norm map)
+    int32_t *counts;        // [nbM*nbN]
+    uint16_t *klist;        // [nbM*nbN*nbK]
+    uint64_t *mask;         // [nbM*nbN*words]
+    MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
+    int32_t *macro_count;   // [n_macro]       entries in the union list
+    int32_t *macro_work;    // [n_macro]       kept products in the macro tile
+    int32_t *order;         // [n_macro]       macro tiles by descending work
+    int64_t *kept_total;    // [1]
+};
+
+hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+                            float *nm, hipStream_t s);
+hipError_t launch_normmap_b(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+                            float *nm, float *nmT, hipStream_t s);
+hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,
+                         uint16_t *out, hipStream_t s);
+hipError_t launch_transpose_normmap(const float *nB, int64_t nbK, int64_t nbN, float *nBt,
+                                    hipStream_t s);
+hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *table,
+                             uint64_t seed, int random, hipStream_t s);
+
+size_t gate_lds_bytes(int tile, int64_t nbK);
+hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
+                       float tau, hipStream_t s);
+
+hipError_t gemm_init();   // one-time kernel attribute set-up
+hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
+                       int64_t K, int64_t N, int tile, float *C, hipStream_t s);
+
+}  // namespace spamm
