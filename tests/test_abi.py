@@ -1,0 +1,79 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every symbol include/spamm.h declares, and reports errors instead of computing."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "spamm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(spamm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = _declared_symbols()
+    for must in ("spamm_create", "spamm_destroy", "spamm_multiply", "spamm_normmap_f32", "spamm_gate",
+                 "spamm_gemm_gated", "spamm_get_mask", "spamm_get_counts", "spamm_get_klist",
+                 "spamm_get_normmap", "spamm_strerror"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol():
+    import cuspamm_amd as sp
+    L = sp.load_library()
+    for name in _declared_symbols():
+        assert hasattr(L, name), name
+    assert L.spamm_version() >= 100
+
+
+def test_struct_layout_matches_header():
+    import cuspamm_amd as sp
+    assert ctypes.sizeof(sp.SpammParams) == 40
+    assert sp.SpammParams.tile.offset == 24 and sp.SpammParams.tau.offset == 28
+    assert ctypes.sizeof(sp.SpammStats) == 40
+
+
+def test_error_strings():
+    import cuspamm_amd as sp
+    L = sp.load_library()
+    seen = set()
+    for code in (0, -1, -2, -3, -4, -5):
+        s = L.spamm_strerror(code).decode()
+        assert s and s != "unknown error"
+        seen.add(s)
+    assert len(seen) == 6
+    assert L.spamm_strerror(-99).decode() == "unknown error"
+
+
+def test_null_arguments_are_rejected_without_a_device():
+    import cuspamm_amd as sp
+    L = sp.load_library()
+    assert L.spamm_create(None, 0) == -1
+    assert L.spamm_destroy(None) == -1
+    assert L.spamm_gate(None, 0.0) == -1
+    assert L.spamm_multiply(None, None, None, None, None) == -1
+
+
+def test_create_without_gpu_reports_no_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    import cuspamm_amd as sp
+    with pytest.raises(sp.SpammError) as ei:
+        sp.SpammContext(0)
+    assert ei.value.code == -5
+
+
+def test_product_package_never_imports_the_oracle():
+    # the checker is test infrastructure: nothing under cuspamm_amd/ may reference it
+    pkg = os.path.join(ROOT, "cuspamm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)
