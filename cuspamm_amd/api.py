@@ -43,7 +43,8 @@ _lib = None
 
 
 def library_path():
-    return os.path.join(HERE, _LIB_NAME)
+    # SPAMM_LIBRARY_PATH lets a developer load an alternative build of the same ABI
+    return os.environ.get("SPAMM_LIBRARY_PATH") or os.path.join(HERE, _LIB_NAME)
 
 
 def load_library():

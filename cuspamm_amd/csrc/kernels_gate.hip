@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     const int words = (nbK + 63) >> 6;
     const int NT = MT * MT;
     uint64_t *lmask = smem;                                   // [NT][words]
-    int *wsum = reinterpret_cast<int *>(smem + (size_t)NT * words);   // [words + 1] prefix
+    int *wsum = reinterpret_cast<int *>(smem + (size_t)NT * words);   // 2 x [words + 1] prefixes
     __shared__ int s_work;
 
     const int lane = threadIdx.x & 63;
@@ -68,34 +68,59 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     if (lane == 0) atomicAdd(&s_work, my_work);
     __syncthreads();
 
-    // ---- phase 2: union list with per-tile bits
+    // ---- phase 2: union list with per-tile bits.  Entries whose k is kept by
+    // every tile of the macro tile ("full") come first, then the partial ones,
+    // each group in ascending k: the GEMM runs a branch-free loop over the
+    // first group.
+    int *wfull = wsum;                       // [words + 1] prefix of full entries
+    int *wpart = wsum + (words + 1);         // [words + 1] prefix of partial entries
     for (int w = threadIdx.x; w < words; w += 256) {
-        uint64_t u = 0;
-        for (int t = 0; t < NT; t++) u |= lmask[(size_t)t * words + w];
-        wsum[w + 1] = __builtin_popcountll(u);
-    }
-    if (threadIdx.x == 0) wsum[0] = 0;
-    __syncthreads();
-    // inclusive scan over words (Hillis-Steele in LDS; words is small)
-    for (int off = 1; off <= words; off <<= 1) {
-        int add[4];
-        int n = 0;
-        for (int w = threadIdx.x; w <= words; w += 256) add[n++] = w >= off ? wsum[w - off] : 0;
-        __syncthreads();
-        n = 0;
-        for (int w = threadIdx.x; w <= words; w += 256) wsum[w] += add[n++];
-        __syncthreads();
-    }
-    for (int k = threadIdx.x; k < nbK; k += 256) {
-        const int w = k >> 6, b = k & 63;
-        uint64_t u = 0, bits = 0;
+        uint64_t u = 0, f = ~0ull;
         for (int t = 0; t < NT; t++) {
             const uint64_t m = lmask[(size_t)t * words + w];
             u |= m;
+            f &= m;
+        }
+        wfull[w + 1] = __builtin_popcountll(f);
+        wpart[w + 1] = __builtin_popcountll(u & ~f);
+    }
+    if (threadIdx.x == 0) { wfull[0] = 0; wpart[0] = 0; }
+    __syncthreads();
+    // inclusive scans over words (Hillis-Steele in LDS; words is small)
+    for (int off = 1; off <= words; off <<= 1) {
+        int addf[4], addp[4];
+        int n = 0;
+        for (int w = threadIdx.x; w <= words; w += 256) {
+            addf[n] = w >= off ? wfull[w - off] : 0;
+            addp[n] = w >= off ? wpart[w - off] : 0;
+            n++;
+        }
+        __syncthreads();
+        n = 0;
+        for (int w = threadIdx.x; w <= words; w += 256) {
+            wfull[w] += addf[n];
+            wpart[w] += addp[n];
+            n++;
+        }
+        __syncthreads();
+    }
+    const int n_full = wfull[words];
+    for (int k = threadIdx.x; k < nbK; k += 256) {
+        const int w = k >> 6, b = k & 63;
+        uint64_t u = 0, f = ~0ull, bits = 0;
+        for (int t = 0; t < NT; t++) {
+            const uint64_t m = lmask[(size_t)t * words + w];
+            u |= m;
+            f &= m;
             bits |= ((m >> b) & 1ull) << t;
         }
         if ((u >> b) & 1ull) {
-            const int pos = wsum[w] + __builtin_popcountll(u & ((1ull << b) - 1ull));
+            const uint64_t below = (1ull << b) - 1ull;
+            int pos;
+            if ((f >> b) & 1ull)
+                pos = wfull[w] + __builtin_popcountll(f & below);
+            else
+                pos = n_full + wpart[w] + __builtin_popcountll(u & ~f & below);
             uint32_t need = 0;
             for (int a = 0; a < MT; a++) {
                 const uint32_t rowbits = (uint32_t)(bits >> (a * MT)) & ((1u << MT) - 1u);
@@ -111,49 +136,57 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         }
     }
     if (threadIdx.x == 0) {
-        g.macro_count[macro] = wsum[words];
+        g.macro_count[2 * macro] = n_full + wpart[words];
+        g.macro_count[2 * macro + 1] = n_full;
         g.macro_work[macro] = s_work;
     }
 }
 
-// Orders macro tiles by descending work (counting sort over quantised work)
-// and totals the kept products.  One workgroup; n_macro is at most a few tens
-// of thousands.
-__global__ __launch_bounds__(1024) void k_order(GateBuffers g, int n_macro, int max_work) {
-    constexpr int NB = 1024;
-    __shared__ int hist[NB];
-    __shared__ int start[NB];
+// Schedule for the GEMM.  Macro tiles are grouped into super tiles of
+// SUPER_M x SUPER_N (= 32, one per CU of an XCD); workgroups are dispatched
+// round-robin over the 8 XCDs, so workgroup b runs on XCD b % 8 and is the
+// (b / 8)-th workgroup that XCD starts.  Each XCD walks a sequence of whole
+// super tiles: the 32 workgroups running together on an XCD (one L2) then
+// share A row panels and B column panels.  Super tiles are ranked by
+// descending kept-product count and dealt to the XCDs in snake order, which
+// balances the XCDs and leaves the lightest super tiles for the tail.
+// One workgroup; O(n^2) ranking over at most a few thousand super tiles.
+__global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
+                                                int n_super) {
+    extern __shared__ int swork[];               // [n_super]
     __shared__ unsigned long long total;
-    for (int b = threadIdx.x; b < NB; b += blockDim.x) hist[b] = 0;
     if (threadIdx.x == 0) total = 0;
     __syncthreads();
     unsigned long long mine = 0;
-    for (int m = threadIdx.x; m < n_macro; m += blockDim.x) {
-        const int wk = g.macro_work[m];
-        mine += (unsigned long long)wk;
-        const int key = (int)(((int64_t)wk * (NB - 1)) / max_work);
-        atomicAdd(&hist[NB - 1 - key], 1);          // bucket 0 = heaviest
+    for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
+        const int sm = sid / nSupN, sn = sid % nSupN;
+        int w = 0;
+        for (int a = 0; a < SUPER_M; a++)
+            for (int b = 0; b < SUPER_N; b++) {
+                const int mi = sm * SUPER_M + a, mj = sn * SUPER_N + b;
+                if (mi < nMacM && mj < nMacN) w += g.macro_work[mi * nMacN + mj];
+            }
+        swork[sid] = w;
+        mine += (unsigned long long)w;
     }
     atomicAdd(&total, mine);
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int acc = 0;
-        for (int b = 0; b < NB; b++) { start[b] = acc; acc += hist[b]; }
-        *g.kept_total = (int64_t)total;
+    for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
+        const int w = swork[sid];
+        int rank = 0;
+        for (int j = 0; j < n_super; j++) {
+            const int wj = swork[j];
+            rank += (wj > w) || (wj == w && j < sid);
+        }
+        g.order[rank] = sid;
     }
-    __syncthreads();
-    for (int m = threadIdx.x; m < n_macro; m += blockDim.x) {
-        const int wk = g.macro_work[m];
-        const int key = (int)(((int64_t)wk * (NB - 1)) / max_work);
-        const int pos = atomicAdd(&start[NB - 1 - key], 1);
-        g.order[pos] = m;
-    }
+    if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;
 }
 
 size_t gate_lds_bytes(int tile, int64_t nbK) {
     const int MT = macro_dim(tile);
     const size_t words = (size_t)((nbK + 63) / 64);
-    return (size_t)MT * MT * words * 8 + (words + 1) * 4 + 8;
+    return (size_t)MT * MT * words * 8 + 2 * (words + 1) * 4 + 8;
 }
 
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
@@ -165,8 +198,9 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     k_gate<<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, MT, nMacN, tau);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int max_work = (int)(MT * MT * nbK);
-    k_order<<<1, 1024, 0, s>>>(g, n_macro, max_work);
+    const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
+    const int n_super = nSupM * nSupN;
+    k_order<<<1, 1024, (size_t)n_super * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super);
     return hipGetLastError();
 }
 

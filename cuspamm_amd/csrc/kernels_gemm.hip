@@ -15,6 +15,10 @@
 // Operands come in the packed layout of spamm_internal.h: a tile's bytes are
 // already in MFMA operand order, so staging is a straight copy and every
 // ds_read_b128 is 512 contiguous bytes per half wave.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "spamm_internal.h"
 
 namespace spamm {
@@ -22,44 +26,58 @@ namespace spamm {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <int B>
 struct GemmCfg {
     static constexpr int SUB = 128 / B;              // tiles per wave per dimension
     static constexpr int MT = 2 * SUB;               // tiles per macro tile per dimension
-    static constexpr int KS = B < 64 ? B : 64;       // k depth of one stage
+    static constexpr int KS = 32;                    // k depth of one stage
     static constexpr int NSPE = B / KS;              // stages per list entry
     static constexpr int SLOT_BYTES = B * KS * 2;    // one tile's share of a stage
     static constexpr int CPS = SLOT_BYTES / 1024;    // 1 KiB wave-loads per slot
-    static constexpr int A_BYTES = MT * SLOT_BYTES;  // 256 rows x KS
-    static constexpr int STAGE_BYTES = 2 * A_BYTES;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int A_BYTES = MT * SLOT_BYTES;  // 256 rows x KS = 16 KiB
+    static constexpr int STAGE_BYTES = 2 * A_BYTES;  // 32 KiB
     static constexpr int TILE_BYTES = B * B * 2;
     static constexpr int RB = B / 32;                // MFMA blocks per tile per dimension
+    static constexpr int CHW = MT * CPS / 4;          // 1 KiB chunks per wave per operand per stage
+    static constexpr int GS = CPS < 4 ? CPS : 4;     // chunks per load group (share a tile)
+    static constexpr int NG = CHW / GS;
+    static constexpr int LPW = 2 * CHW;              // load instructions per wave per stage
 };
 
-#define SPAMM_WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)
+// s_waitcnt immediates (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | 0x70 | ((lgkm & 15) << 8); }
 
-// 16 bytes per lane straight from global memory into LDS: lane l's vector
-// lands at lds_addr + 16*l.  Written as inline assembly so that the compiler's
-// wait-count insertion does not see an LDS write it cannot disambiguate (it
-// would put a full vmcnt(0) wait before every LDS read and serialise the
-// double buffering); completion is awaited explicitly with
-// SPAMM_WAIT_VMCNT0() before the workgroup barrier.  M0 carries the LDS
-// address; nothing else in this kernel keeps a value in M0.
-__device__ __forceinline__ void dma16(const void *gsrc, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+// One 1 KiB wave-load straight from global memory into LDS: lane l's 16 bytes
+// land at lds_addr + IMM + 16*l, read from sbase + IMM + voff (the instruction
+// offset applies to the global and to the LDS address alike).  Written as
+// inline assembly so that the compiler's wait-count insertion does not see an
+// LDS write it cannot disambiguate (it would put a full vmcnt(0) wait before
+// every LDS read and serialise the staging ring); completion is awaited
+// explicitly with s_waitcnt vmcnt before the workgroup barrier.  M0 carries
+// the LDS address; nothing else in this kernel keeps a value in M0.
+template <int IMM>
+__device__ __forceinline__ void dma_load(const unsigned char *sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
                  :
-                 : "s"(lds_addr), "v"(gsrc)
+                 : "s"(lds_addr), "v"(voff), "s"(sbase), "n"(IMM)
                  : "memory");
 }
 
-template <int B>
+// One workgroup per macro tile.  The k loop walks stages of 32 k (a list entry
+// is B/32 stages); stage t lives in LDS buffer t % NBUF.  Ring protocol, with
+// "sync(t)" = every wave waits for its own loads of stage t+1, then a
+// workgroup barrier: after sync(t) stage t+1 is readable by all waves and no
+// wave reads stage t any more, so the loads of stage t+NBUF go into stage t's
+// buffer.  NBUF-1 stages are in flight while one is multiplied.
+template <int B, int NBUF>
 __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ pA,
                                               const unsigned char *__restrict__ pB,
                                               const MacroEntry *__restrict__ macro_list,
                                               const int32_t *__restrict__ macro_count,
-                                              const int32_t *__restrict__ order, int nbM, int nbK,
+                                              const int32_t *__restrict__ order,
+                                              int n_super, int nSupN, int nMacM, int nbM, int nbK,
                                               int nbN, int nMacN, int64_t M, int64_t N,
                                               float *__restrict__ C) {
     using G = GemmCfg<B>;
@@ -69,13 +87,34 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
-    const int macro = __builtin_amdgcn_readfirstlane(order[blockIdx.x]);
-    const int mi = macro / nMacN, mj = macro % nMacN;
-    const int U = __builtin_amdgcn_readfirstlane(macro_count[macro]);
+    // Workgroup b runs on XCD b % NUM_XCD and is that XCD's (b / NUM_XCD)-th
+    // workgroup; every XCD walks whole super tiles (32 macro tiles that share
+    // operand panels), dealt out by descending work in snake order.
+    const int xcd = blockIdx.x % NUM_XCD, pos = blockIdx.x / NUM_XCD;
+    constexpr int SUPER = SUPER_M * SUPER_N;
+    const int round = pos / SUPER, slot = pos % SUPER;
+    const int srank = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - xcd : xcd);
+    if (srank >= n_super) return;
+    const int sid = __builtin_amdgcn_readfirstlane(order[srank]);
+    const int mi = (sid / nSupN) * SUPER_M + slot / SUPER_N, mj = (sid % nSupN) * SUPER_N + slot % SUPER_N;
+    if (mi >= nMacM || mj >= nMacN) return;
+    const int macro = mi * nMacN + mj;
+    const int U = __builtin_amdgcn_readfirstlane(macro_count[2 * macro]);
+    const int Ufull = __builtin_amdgcn_readfirstlane(macro_count[2 * macro + 1]);
     entry_ptr ents = (entry_ptr)(uintptr_t)(macro_list + (int64_t)macro * nbK);
-    const int S = U * G::NSPE;
+    const int S = U * G::NSPE, Sfull = Ufull * G::NSPE;
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+    if (S == 0) {
+        // nothing kept in this macro tile: C still has to be overwritten with zeros
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int64_t r0 = (int64_t)mi * 256, c0 = (int64_t)mj * 256 + lane * 4;
+        if (c0 < N)
+            for (int r = wave; r < 256 && r0 + r < M; r += 4)
+                *reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0) = zero;
+        return;
+    }
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -85,105 +124,222 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[r][c][i] = 0.0f;
 
-    // Stage s -> LDS buffer s&1.  Each wave copies CHW consecutive 1 KiB
-    // chunks of the A part and of the B part.
-    auto issue_loads = [&](int s, u32x4 en) {
-        const int h = s % G::NSPE;
-        const uint32_t k = en.x, need = en.y;
-        const uint32_t buf = lds_base + (s & 1) * G::STAGE_BYTES;
-        constexpr int CHW = G::MT * G::CPS / 4;
+    {
+        // ---- staging: each wave copies CHW consecutive 1 KiB chunks of the A
+        // part and of the B part of a stage, in groups of GS chunks that share
+        // a tile.  Tiles beyond the matrix edge are clamped to the last tile
+        // row / column (loaded but never multiplied) and stages beyond the
+        // last are clamped to the last (loaded but never read), so staging is
+        // branch-free and the number of loads in flight is always the same.
+        static_assert(G::LPW == 8, "the issue schedule below assumes 8 loads per wave per stage");
+        const unsigned char *rowA[G::NG], *rowB[G::NG];
+        uint32_t ldsA[G::NG];
 #pragma unroll
-        for (int c = 0; c < CHW; c++) {
-            const int chunk = wave * CHW + c;
-            const int slot = chunk / G::CPS, within = chunk % G::CPS;
-            if ((need >> slot) & 1u) {
-                const unsigned char *src = pA + ((int64_t)(mi * G::MT + slot) * nbK + k) * G::TILE_BYTES +
-                                           h * G::SLOT_BYTES + within * 1024 + lane * 16;
-                dma16(src, buf + slot * G::SLOT_BYTES + within * 1024);
-            }
+        for (int g = 0; g < G::NG; g++) {
+            const int chunk0 = wave * G::CHW + g * G::GS;
+            const int slot = chunk0 / G::CPS, within0 = chunk0 % G::CPS;
+            int ti = mi * G::MT + slot, tj = mj * G::MT + slot;
+            ti = ti < nbM ? ti : nbM - 1;
+            tj = tj < nbN ? tj : nbN - 1;
+            rowA[g] = pA + (int64_t)ti * nbK * G::TILE_BYTES + within0 * 1024;
+            rowB[g] = pB + (int64_t)tj * nbK * G::TILE_BYTES + within0 * 1024;
+            ldsA[g] = lds_base + slot * G::SLOT_BYTES + within0 * 1024;
         }
-#pragma unroll
-        for (int c = 0; c < CHW; c++) {
-            const int chunk = wave * CHW + c;
-            const int slot = chunk / G::CPS, within = chunk % G::CPS;
-            if ((need >> (8 + slot)) & 1u) {
-                const unsigned char *src = pB + ((int64_t)(mj * G::MT + slot) * nbK + k) * G::TILE_BYTES +
-                                           h * G::SLOT_BYTES + within * 1024 + lane * 16;
-                dma16(src, buf + G::A_BYTES + slot * G::SLOT_BYTES + within * 1024);
-            }
-        }
-    };
+        const uint32_t voff = lane * 16;
 
-    // LDS byte offset (inside the A or B part of a stage) of this lane's
-    // operand vector for MFMA block `blk` (32 of the wave's 128 rows/columns)
-    // at k step kk.
-    auto frag_off = [&](int wsel, int blk, int kk) -> int {
-        const int slot = wsel * G::SUB + (blk * 32) / B;
-        const int ro = (blk * 32) % B;
-        return slot * G::SLOT_BYTES + (((2 * kk + (lane >> 5)) * B) + ro + (lane & 31)) * 16;
-    };
+        auto stage_k = [&](int t) -> uint32_t {
+            const int tc = t < S ? t : S - 1;
+            return ents[tc / G::NSPE].x;
+        };
+        // Load i (0..LPW-1) of a stage: i < CHW are the wave's A chunks, the
+        // rest its B chunks.  A wave is in-order and alone on its SIMD, so a
+        // burst of loads that backs up the address FIFO stalls its MFMAs; the
+        // loops below therefore issue one load every few MFMAs.
+        struct StageAddr {
+            int64_t koff;
+            uint32_t boff;
+        };
+        auto stage_addr = [&](int t, uint32_t k) -> StageAddr {
+            const int tc = t < S ? t : S - 1;
+            StageAddr sa;
+            sa.koff = (int64_t)k * G::TILE_BYTES + (tc % G::NSPE) * G::SLOT_BYTES;
+            sa.boff = (uint32_t)(t % NBUF) * G::STAGE_BYTES;
+            return sa;
+        };
+        auto issue_one = [&](const StageAddr &sa, auto idx) {
+            constexpr int i = decltype(idx)::value;
+            constexpr int op = i / G::CHW, ci = i % G::CHW;
+            constexpr int g = ci / G::GS, j = ci % G::GS;
+            if constexpr (op == 0)
+                dma_load<j * 1024>(rowA[g] + sa.koff, voff, ldsA[g] + sa.boff);
+            else
+                dma_load<j * 1024>(rowB[g] + sa.koff, voff, ldsA[g] + G::A_BYTES + sa.boff);
+        };
+#define SPAMM_ISSUE(sa, i) issue_one(sa, std::integral_constant<int, i>{})
+        auto issue_all = [&](const StageAddr &sa) {
+            SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); SPAMM_ISSUE(sa, 2); SPAMM_ISSUE(sa, 3);
+            SPAMM_ISSUE(sa, 4); SPAMM_ISSUE(sa, 5); SPAMM_ISSUE(sa, 6); SPAMM_ISSUE(sa, 7);
+        };
+        auto issue_head = [&](const StageAddr &sa) { SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); };
+        auto issue_tail = [&](const StageAddr &sa) {
+            SPAMM_ISSUE(sa, 2); SPAMM_ISSUE(sa, 3); SPAMM_ISSUE(sa, 4);
+            SPAMM_ISSUE(sa, 5); SPAMM_ISSUE(sa, 6); SPAMM_ISSUE(sa, 7);
+        };
+        // every wave: own loads of the next stage landed and own LDS reads
+        // done; then the barrier makes both true for the whole workgroup
+        auto sync_next = [&]() {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2), 0));
+            __syncthreads();
+        };
 
-    u32x4 cur = {0, 0, 0, 0};
-    if (S > 0) {
-        cur = ents[0];
-        issue_loads(0, cur);
-    }
-    for (int s = 0; s < S; s++) {
-        u32x4 nxt = cur;
-        if (s + 1 < S) nxt = ents[(s + 1) / G::NSPE];
-        SPAMM_WAIT_VMCNT0();
-        __syncthreads();
-        if (s + 1 < S) issue_loads(s + 1, nxt);
-
-        // bits of this wave's SUB x SUB tiles
-        const uint64_t mask = ((uint64_t)cur.w << 32) | cur.z;
-        uint32_t sb = 0;
-#pragma unroll
-        for (int a = 0; a < G::SUB; a++)
-#pragma unroll
-            for (int b = 0; b < G::SUB; b++) {
-                const int bit = (wr * G::SUB + a) * G::MT + wc * G::SUB + b;
-                sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
-            }
-
-        if (sb != 0) {
-            const unsigned char *bufA = smem + (s & 1) * G::STAGE_BYTES;
+        // LDS byte offset (inside the A or B part of a stage) of this lane's
+        // operand vector for MFMA block `blk` (32 of the wave's 128
+        // rows/columns) at k step kk (0 or 1) of the stage.
+        auto frag_off = [&](int wsel, int blk, int kk) -> int {
+            const int slot = wsel * G::SUB + (blk * 32) / B;
+            const int ro = (blk * 32) % B;
+            return slot * G::SLOT_BYTES + (((2 * kk + (lane >> 5)) * B) + ro + (lane & 31)) * 16;
+        };
+        auto load_frags = [&](half8 (&af)[4], half8 (&bf)[4], int t, int kk) {
+            const unsigned char *bufA = smem + (t % NBUF) * G::STAGE_BYTES;
             const unsigned char *bufB = bufA + G::A_BYTES;
-            constexpr int NKK = G::KS / 16;
-            half8 af[2][4], bf[2][4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) af[0][r] = *reinterpret_cast<const half8 *>(bufA + frag_off(wr, r, 0));
+            for (int r = 0; r < 4; r++) af[r] = *reinterpret_cast<const half8 *>(bufA + frag_off(wr, r, kk));
 #pragma unroll
-            for (int c = 0; c < 4; c++) bf[0][c] = *reinterpret_cast<const half8 *>(bufB + frag_off(wc, c, 0));
+            for (int c = 0; c < 4; c++) bf[c] = *reinterpret_cast<const half8 *>(bufB + frag_off(wc, c, kk));
+        };
+
+        // ---- prologue: stages 0..NBUF-2 and the first two loads of stage
+        // NBUF-1 (the "head"; its "tail" of six follows inside the loops, and
+        // so on for every later stage); wait for stage 0
 #pragma unroll
-            for (int kk = 0; kk < NKK; kk++) {
-                if (kk + 1 < NKK) {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        af[(kk + 1) & 1][r] = *reinterpret_cast<const half8 *>(bufA + frag_off(wr, r, kk + 1));
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        bf[(kk + 1) & 1][c] = *reinterpret_cast<const half8 *>(bufB + frag_off(wc, c, kk + 1));
+        for (int t = 0; t < NBUF - 1; t++) issue_all(stage_addr(t, stage_k(t)));
+        StageAddr sa_tail = stage_addr(NBUF - 1, stage_k(NBUF - 1));
+        issue_head(sa_tail);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2) + 2, 0));
+        __syncthreads();
+
+        int t = 0;
+        // ---- loop 1: entries kept by all tiles of the macro tile; no
+        // branches.  Operand vectors are double buffered in registers (a0/b0:
+        // k step 0, a1/b1: k step 1) and every LDS read is issued 8+ MFMAs
+        // before its first use.  The sync sits in the middle of k step 1 so
+        // that the first LDS reads of the next stage overlap its second half.
+        // Global->LDS loads are spread out: one after every fourth MFMA.
+        // sched_barrier(0) pins the issue order written here.
+#define SPAMM_MFMA(A, Bv, r, c) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[r], Bv[c], acc[r][c], 0, 0, 0)
+#define SPAMM_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define SPAMM_LDA(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufA + frag_off(wr, blk, kk))
+#define SPAMM_LDB(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufB + frag_off(wc, blk, kk))
+        if (Sfull > 0) {
+            half8 a0[4], b0[4], a1[4], b1[4];
+            load_frags(a0, b0, 0, 0);
+            uint32_t knext = stage_k(NBUF);
+            for (; t < Sfull; t++) {
+                const uint32_t kissue = knext;
+                {
+                    const unsigned char *bufA = smem + (t % NBUF) * G::STAGE_BYTES;
+                    const unsigned char *bufB = bufA + G::A_BYTES;
+                    // k step 0 (16 MFMA) with the 8 reads of k step 1 in between
+                    SPAMM_MFMA(a0, b0, 0, 0); SPAMM_MFMA(a0, b0, 0, 1); SPAMM_LDA(a1[0], 0, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 0, 2); SPAMM_MFMA(a0, b0, 0, 3); SPAMM_LDB(b1[0], 0, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 2); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 1, 0); SPAMM_MFMA(a0, b0, 1, 1); SPAMM_LDB(b1[1], 1, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 1, 2); SPAMM_MFMA(a0, b0, 1, 3); SPAMM_LDB(b1[2], 2, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 3); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 2, 0); SPAMM_MFMA(a0, b0, 2, 1); SPAMM_LDB(b1[3], 3, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 2, 2); SPAMM_MFMA(a0, b0, 2, 3); SPAMM_LDA(a1[1], 1, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 4); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 3, 0); SPAMM_MFMA(a0, b0, 3, 1); SPAMM_LDA(a1[2], 2, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 3, 2); SPAMM_MFMA(a0, b0, 3, 3); SPAMM_LDA(a1[3], 3, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 5); SPAMM_FENCE();
+                    // first half of k step 1
+                    SPAMM_MFMA(a1, b1, 0, 0); SPAMM_MFMA(a1, b1, 0, 1); SPAMM_MFMA(a1, b1, 0, 2); SPAMM_MFMA(a1, b1, 0, 3);
+                    SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 6); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 1, 0); SPAMM_MFMA(a1, b1, 1, 1); SPAMM_MFMA(a1, b1, 1, 2); SPAMM_MFMA(a1, b1, 1, 3);
+                    SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 7); SPAMM_FENCE();
                 }
-#pragma unroll
-                for (int a = 0; a < G::SUB; a++)
-#pragma unroll
-                    for (int b = 0; b < G::SUB; b++) {
-                        if ((sb >> (a * G::SUB + b)) & 1u) {
-#pragma unroll
-                            for (int r = 0; r < G::RB; r++)
-#pragma unroll
-                                for (int c = 0; c < G::RB; c++)
-                                    acc[a * G::RB + r][b * G::RB + c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                                        af[kk & 1][a * G::RB + r], bf[kk & 1][b * G::RB + c],
-                                        acc[a * G::RB + r][b * G::RB + c], 0, 0, 0);
-                        }
-                    }
+                sync_next();
+                SPAMM_FENCE();
+                // scalar load placed here so that no LDS wait follows it closely
+                knext = stage_k(t + 1 + NBUF);
+                sa_tail = stage_addr(t + NBUF, kissue);
+                SPAMM_FENCE();
+                {
+                    const unsigned char *bufA = smem + ((t + 1) % NBUF) * G::STAGE_BYTES;
+                    const unsigned char *bufB = bufA + G::A_BYTES;
+                    // second half of k step 1 with the 8 reads of the next stage's k step 0
+                    SPAMM_MFMA(a1, b1, 2, 0); SPAMM_LDA(a0[0], 0, 0); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 2, 1); SPAMM_LDB(b0[0], 0, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 2, 2); SPAMM_LDB(b0[1], 1, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 2, 3); SPAMM_LDB(b0[2], 2, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 3, 0); SPAMM_LDB(b0[3], 3, 0); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 3, 1); SPAMM_LDA(a0[1], 1, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 3, 2); SPAMM_LDA(a0[2], 2, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 3, 3); SPAMM_LDA(a0[3], 3, 0); SPAMM_FENCE();
+                }
             }
         }
-        cur = nxt;
+        // ---- loop 2: entries kept by some tiles only; a wave multiplies
+        // exactly the (tile row, tile column) pairs whose bit is set
+        for (; t < S; t++) {
+            const uint32_t knext = stage_k(t + NBUF);
+            issue_tail(sa_tail);
+            const u32x4 cur = ents[t / G::NSPE];
+            const uint64_t mask = ((uint64_t)cur.w << 32) | cur.z;
+            uint32_t sb = 0;
+#pragma unroll
+            for (int a = 0; a < G::SUB; a++)
+#pragma unroll
+                for (int b = 0; b < G::SUB; b++) {
+                    const int bit = (wr * G::SUB + a) * G::MT + wc * G::SUB + b;
+                    sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
+                }
+#ifdef SPAMM_EXP_NOLOOP2
+            sb = 0;
+#endif
+            if (sb != 0) {
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++) {
+                    half8 af[4], bf[4];
+                    load_frags(af, bf, t, kk);
+#pragma unroll
+                    for (int a = 0; a < G::SUB; a++)
+#pragma unroll
+                        for (int b = 0; b < G::SUB; b++) {
+                            if ((sb >> (a * G::SUB + b)) & 1u) {
+#pragma unroll
+                                for (int r = 0; r < G::RB; r++)
+#pragma unroll
+                                    for (int c = 0; c < G::RB; c++)
+                                        acc[a * G::RB + r][b * G::RB + c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                                            af[a * G::RB + r], bf[b * G::RB + c], acc[a * G::RB + r][b * G::RB + c], 0,
+                                            0, 0);
+                            }
+                        }
+                }
+            }
+            sync_next();
+            sa_tail = stage_addr(t + NBUF, knext);
+            issue_head(sa_tail);
+        }
+#undef SPAMM_MFMA
+#undef SPAMM_FENCE
+#undef SPAMM_LDA
+#undef SPAMM_LDB
+#undef SPAMM_ISSUE
+        // the ring still holds clamped loads: let them land before the
+        // workgroup gives its LDS back
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     }
 
+#ifdef SPAMM_EXP_NOEPI
+    if (acc[0][0][0] != 12345.0f) return;
+#endif
     // ---- epilogue: C[row, col], row-major, ld N (cuSpAMM.cu:391).  MFMA
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
     // column l%32 of the block.
@@ -200,19 +356,51 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             for (int i = 0; i < 16; i++) out[(int64_t)(8 * (i / 4) + (i % 4)) * N] = acc[r][c][i];
         }
     }
+
+}
+
+static int g_nbuf = 4;
+
+template <int B, int NBUF>
+static hipError_t set_lds_attr() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, NBUF>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, NBUF * GemmCfg<B>::STAGE_BYTES);
 }
 
 hipError_t gemm_init() {
+    const char *env = getenv("SPAMM_GEMM_NBUF");     // developer tuning knob: depth of the LDS ring
+    if (env && (env[0] == '3' || env[0] == '4' || env[0] == '5')) g_nbuf = env[0] - '0';
     hipError_t e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<32>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, GemmCfg<32>::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<64>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, GemmCfg<64>::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<128>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, GemmCfg<128>::LDS_BYTES);
-    return e;
+    if ((e = set_lds_attr<32, 3>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<32, 4>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<32, 5>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<64, 3>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<64, 4>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<64, 5>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<128, 3>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<128, 4>()) != hipSuccess) return e;
+    if ((e = set_lds_attr<128, 5>()) != hipSuccess) return e;
+    return hipSuccess;
+}
+
+template <int B, int NBUF>
+static void launch_one(unsigned grid, const unsigned char *pA, const unsigned char *pB, const GateBuffers &g,
+                       int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C, hipStream_t s) {
+    const int MT = GemmCfg<B>::MT;
+    const int nMacM = (nbM + MT - 1) / MT;
+    const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
+    k_gemm<B, NBUF><<<grid, 256, NBUF * GemmCfg<B>::STAGE_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count, g.order,
+                                                                     nSupM * nSupN, nSupN, nMacM, nbM, nbK, nbN,
+                                                                     nMacN, M, N, C);
+}
+
+template <int B>
+static void launch_tile(int nbuf, unsigned grid, const unsigned char *pA, const unsigned char *pB,
+                        const GateBuffers &g, int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C,
+                        hipStream_t s) {
+    if (nbuf == 3) launch_one<B, 3>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
+    else if (nbuf == 5) launch_one<B, 5>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
+    else launch_one<B, 4>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
 }
 
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
@@ -220,23 +408,15 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
-    const unsigned grid = (unsigned)(nMacM * nMacN);
+    const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
+    const int rounds = (nSupM * nSupN + NUM_XCD - 1) / NUM_XCD;
+    const unsigned grid = (unsigned)(rounds * NUM_XCD * SUPER_M * SUPER_N);
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
     switch (tile) {
-        case 32:
-            k_gemm<32><<<grid, 256, GemmCfg<32>::LDS_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count,
-                                                               g.order, nbM, nbK, nbN, nMacN, M, N, C);
-            break;
-        case 64:
-            k_gemm<64><<<grid, 256, GemmCfg<64>::LDS_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count,
-                                                               g.order, nbM, nbK, nbN, nMacN, M, N, C);
-            break;
-        case 128:
-            k_gemm<128><<<grid, 256, GemmCfg<128>::LDS_BYTES, s>>>(pA, pB, g.macro_list,
-                                                                 g.macro_count, g.order, nbM, nbK, nbN, nMacN,
-                                                                 M, N, C);
-            break;
+        case 32: launch_tile<32>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 64: launch_tile<64>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 128: launch_tile<128>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

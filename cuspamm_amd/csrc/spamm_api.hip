@@ -267,10 +267,10 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->klist, nt * s.nbK * 2))) return rc;
     if ((rc = ensure(c, c->mask, nt * s.words * 8))) return rc;
     if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
-    if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 4))) return rc;
+    if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
     if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
     if ((rc = ensure(c, c->order, (size_t)s.n_macro * 4))) return rc;
-    if ((rc = ensure(c, c->kept_total, 8))) return rc;
+    if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
     HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[3], c->stream)); c->ev_gate = true; }

@@ -24,6 +24,13 @@ namespace spamm {
 // (256 x 256 elements); one workgroup of the gated GEMM owns one macro tile.
 inline int macro_dim(int tile) { return 256 / tile; }
 
+// Macro tiles are scheduled in super tiles of SUPER_M x SUPER_N macro tiles:
+// 32 workgroups, one per CU of an XCD, that share operand panels in that
+// XCD's L2.
+constexpr int SUPER_M = 4;
+constexpr int SUPER_N = 8;
+constexpr int NUM_XCD = 8;
+
 // One entry of a macro tile's union k list: tile column/row k of the
 // operands plus the set of output tiles (bit a*MT+b = tile row a, column b of
 // the macro tile) that keep the product with this k.  16 bytes so that the
@@ -42,10 +49,10 @@ struct GateBuffers {
     uint16_t *klist;        // [nbM*nbN*nbK]
     uint64_t *mask;         // [nbM*nbN*words]
     MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
-    int32_t *macro_count;   // [n_macro]       entries in the union list
+    int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
     int32_t *macro_work;    // [n_macro]       kept products in the macro tile
-    int32_t *order;         // [n_macro]       macro tiles by descending work
-    int64_t *kept_total;    // [1]
+    int32_t *order;         // [n_super]       super tiles by descending work
+    int64_t *kept_total;    // [1]  kept products
 };
 
 hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
