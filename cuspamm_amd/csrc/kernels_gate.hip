@@ -105,6 +105,31 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         __syncthreads();
     }
     const int n_full = wfull[words];
+    const int n_part = wpart[words];
+    // Each group is rotated to start at an anchor k shared by the whole super
+    // tile (the k where its diagonal would sit): the workgroups of a super
+    // tile run together on one XCD, and walking k from a common start keeps
+    // them on the same A row panels and B column panels at the same time.
+    int rot_f = 0, rot_p = 0;              // entries of each group below the anchor
+    {
+        const int mMT = nMacN > 0 ? MT : MT;
+        const int sm = mi / SUPER_M, sn = mj / SUPER_N;
+        const float ic = ((sm * SUPER_M + 0.5f * SUPER_M) * mMT) / (float)nbM;
+        const float jc = ((sn * SUPER_N + 0.5f * SUPER_N) * mMT) / (float)nbN;
+        float fa = 0.5f * (ic + jc) * (float)nbK - 0.5f * SUPER_N * mMT;
+        int anchor = (int)fa;
+        anchor = anchor < 0 ? 0 : (anchor > nbK - 1 ? nbK - 1 : anchor);
+        const int wa = anchor >> 6, ba = anchor & 63;
+        uint64_t u = 0, f = ~0ull;
+        for (int t = 0; t < NT; t++) {
+            const uint64_t m = lmask[(size_t)t * words + wa];
+            u |= m;
+            f &= m;
+        }
+        const uint64_t below = (1ull << ba) - 1ull;
+        rot_f = wfull[wa] + __builtin_popcountll(f & below);
+        rot_p = wpart[wa] + __builtin_popcountll(u & ~f & below);
+    }
     for (int k = threadIdx.x; k < nbK; k += 256) {
         const int w = k >> 6, b = k & 63;
         uint64_t u = 0, f = ~0ull, bits = 0;
@@ -117,10 +142,14 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         if ((u >> b) & 1ull) {
             const uint64_t below = (1ull << b) - 1ull;
             int pos;
-            if ((f >> b) & 1ull)
-                pos = wfull[w] + __builtin_popcountll(f & below);
-            else
-                pos = n_full + wpart[w] + __builtin_popcountll(u & ~f & below);
+            if ((f >> b) & 1ull) {
+                pos = wfull[w] + __builtin_popcountll(f & below) - rot_f;
+                if (pos < 0) pos += n_full;
+            } else {
+                pos = wpart[w] + __builtin_popcountll(u & ~f & below) - rot_p;
+                if (pos < 0) pos += n_part;
+                pos += n_full;
+            }
             uint32_t need = 0;
             for (int a = 0; a < MT; a++) {
                 const uint32_t rowbits = (uint32_t)(bits >> (a * MT)) & ((1u << MT) - 1u);
@@ -136,7 +165,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         }
     }
     if (threadIdx.x == 0) {
-        g.macro_count[2 * macro] = n_full + wpart[words];
+        g.macro_count[2 * macro] = n_full + n_part;
         g.macro_count[2 * macro + 1] = n_full;
         g.macro_work[macro] = s_work;
     }
@@ -145,31 +174,49 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // Schedule for the GEMM.  Macro tiles are grouped into super tiles of
 // SUPER_M x SUPER_N (= 32, one per CU of an XCD); workgroups are dispatched
 // round-robin over the 8 XCDs, so workgroup b runs on XCD b % 8 and is the
-// (b / 8)-th workgroup that XCD starts.  Each XCD walks a sequence of whole
-// super tiles: the 32 workgroups running together on an XCD (one L2) then
-// share A row panels and B column panels.  Super tiles are ranked by
-// descending kept-product count and dealt to the XCDs in snake order, which
-// balances the XCDs and leaves the lightest super tiles for the tail.
+// (b / 8)-th workgroup that XCD starts.
+//   1. Super tiles are ranked by descending kept-product count and dealt to
+//      the XCDs in snake order: every XCD owns whole super tiles, so the
+//      workgroups sharing one L2 share A row panels and B column panels, and
+//      the XCDs get equal work.
+//   2. Inside an XCD the macro tiles are ordered by work level (SCHED_LEVELS
+//      classes of the kept-product count, heaviest first) and, inside a
+//      level, in super-tile order.  A free CU always takes the next workgroup
+//      in order, so heaviest-first keeps the tail short (list scheduling),
+//      while neighbours of one level are still neighbours in the matrix.
+//   3. Macro tiles with nothing kept come last in each XCD's sequence; the
+//      computing workgroups zero-fill them after their own epilogue.
+// Output: order[x * P + q] = macro tile id of XCD x's q-th workgroup,
+// sched[x] = number of computing items, sched[8 + x] = number of all items.
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
-                                                int n_super) {
-    extern __shared__ int swork[];               // [n_super]
+                                                int n_super, int rounds) {
+    extern __shared__ int swork[];               // [n_super] work, then reused: [n_super] id by rank
+    int *srank_id = swork + n_super;
     __shared__ unsigned long long total;
-    if (threadIdx.x == 0) total = 0;
+    __shared__ int maxwork;
+    const int P = rounds * SUPER_M * SUPER_N;
+    if (threadIdx.x == 0) { total = 0; maxwork = 1; }
     __syncthreads();
     unsigned long long mine = 0;
+    int mymax = 0;
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int sm = sid / nSupN, sn = sid % nSupN;
         int w = 0;
         for (int a = 0; a < SUPER_M; a++)
             for (int b = 0; b < SUPER_N; b++) {
                 const int mi = sm * SUPER_M + a, mj = sn * SUPER_N + b;
-                if (mi < nMacM && mj < nMacN) w += g.macro_work[mi * nMacN + mj];
+                if (mi < nMacM && mj < nMacN) {
+                    const int mw = g.macro_work[mi * nMacN + mj];
+                    w += mw;
+                    mymax = mw > mymax ? mw : mymax;
+                }
             }
         swork[sid] = w;
         mine += (unsigned long long)w;
     }
     atomicAdd(&total, mine);
+    atomicMax(&maxwork, mymax);
     __syncthreads();
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int w = swork[sid];
@@ -178,7 +225,76 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
             const int wj = swork[j];
             rank += (wj > w) || (wj == w && j < sid);
         }
-        g.order[rank] = sid;
+        srank_id[rank] = sid;
+    }
+    for (int i = threadIdx.x; i < NUM_XCD * P; i += blockDim.x) g.order[i] = -1;
+    __syncthreads();
+
+    // item of XCD x at raw position p (round-major, then slot), or -1; level of that item
+    const int mw_max = maxwork;
+    auto item_at = [&](int x, int p, int &level) -> int {
+        const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
+        const int sr = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - x : x);
+        if (sr >= n_super) return -1;
+        const int sid = srank_id[sr];
+        const int mi = (sid / nSupN) * SUPER_M + slot / SUPER_N, mj = (sid % nSupN) * SUPER_N + slot % SUPER_N;
+        if (mi >= nMacM || mj >= nMacN) return -1;
+        const int m = mi * nMacN + mj;
+        const int mw = g.macro_work[m];
+        level = mw > 0 ? 1 + (int)(((int64_t)(mw - 1) * (SCHED_LEVELS - 1)) / mw_max) : 0;
+        return m;
+    };
+    // raw sequence (round-major, slot-minor) with the level in the top byte, in the upper half of `order`
+    int32_t *raw = g.order + NUM_XCD * P;
+    for (int i = threadIdx.x; i < NUM_XCD * P; i += blockDim.x) {
+        int level = 0;
+        const int m = item_at(i / P, i % P, level);
+        raw[i] = m >= 0 ? (m | (level << 24)) : -1;
+    }
+    __syncthreads();
+    // one wave per XCD: count per level, prefix (heaviest level first, empty tiles last), stable scatter
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (wave < NUM_XCD) {
+        const int x = wave;
+        const int32_t *rx = raw + x * P;
+        int mycnt = 0;                       // lane lv < SCHED_LEVELS keeps the count of level lv
+        for (int p0 = 0; p0 < P; p0 += 64) {
+            const int p = p0 + lane;
+            const int v = p < P ? rx[p] : -1;
+            const int level = v >= 0 ? (v >> 24) : -1;
+#pragma unroll
+            for (int lv = 0; lv < SCHED_LEVELS; lv++) {
+                const int c = __builtin_popcountll(__ballot(level == lv));
+                if (lane == lv) mycnt += c;
+            }
+        }
+        // exclusive prefix over levels in descending order: base(lv) = sum of counts of levels > lv
+        int base = 0, ncomp = 0, nall = 0;
+#pragma unroll
+        for (int lv = SCHED_LEVELS - 1; lv >= 0; lv--) {
+            const int c = __shfl(mycnt, lv, 64);
+            if (lane == lv) base = nall;
+            if (lv == 0) ncomp = nall;
+            nall += c;
+        }
+        if (lane == 0) {
+            g.sched[x] = ncomp;
+            g.sched[NUM_XCD + x] = nall;
+        }
+        for (int p0 = 0; p0 < P; p0 += 64) {
+            const int p = p0 + lane;
+            const int v = p < P ? rx[p] : -1;
+            const int level = v >= 0 ? (v >> 24) : -1;
+            int pos = -1;
+#pragma unroll
+            for (int lv = 0; lv < SCHED_LEVELS; lv++) {
+                const uint64_t bal = __ballot(level == lv);
+                const int b0 = __shfl(base, lv, 64);
+                if (level == lv) pos = b0 + __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+                if (lane == lv) base += __builtin_popcountll(bal);
+            }
+            if (pos >= 0) g.order[x * P + pos] = v & 0xffffff;
+        }
     }
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;
 }
@@ -200,7 +316,8 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     if (e != hipSuccess) return e;
     const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
     const int n_super = nSupM * nSupN;
-    k_order<<<1, 1024, (size_t)n_super * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super);
+    const int rounds = (n_super + NUM_XCD - 1) / NUM_XCD;
+    k_order<<<1, 1024, (size_t)n_super * 2 * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super, rounds);
     return hipGetLastError();
 }
 

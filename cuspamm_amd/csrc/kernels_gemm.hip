@@ -28,6 +28,13 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+#ifdef SPAMM_EXP_TRACE
+__device__ unsigned long long g_trace[16384 * 8];
+#define SPAMM_TRACE(slot) do { if (threadIdx.x == 0) { g_trace[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64(); if ((slot) == 1) g_trace[(size_t)blockIdx.x * 8 + 7] = clock64(); if ((slot) == 2) g_trace[(size_t)blockIdx.x * 8 + 7] = clock64() - g_trace[(size_t)blockIdx.x * 8 + 7]; } } while (0)
+#else
+#define SPAMM_TRACE(slot) do { } while (0)
+#endif
+
 template <int B>
 struct GemmCfg {
     static constexpr int SUB = 128 / B;              // tiles per wave per dimension
@@ -77,8 +84,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                                               const MacroEntry *__restrict__ macro_list,
                                               const int32_t *__restrict__ macro_count,
                                               const int32_t *__restrict__ order,
-                                              int n_super, int nSupN, int nMacM, int nbM, int nbK,
-                                              int nbN, int nMacN, int64_t M, int64_t N,
+                                              const int32_t *__restrict__ sched, int P, int nbM,
+                                              int nbK, int nbN, int nMacN, int64_t M, int64_t N,
                                               float *__restrict__ C) {
     using G = GemmCfg<B>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -87,18 +94,19 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
-    // Workgroup b runs on XCD b % NUM_XCD and is that XCD's (b / NUM_XCD)-th
-    // workgroup; every XCD walks whole super tiles (32 macro tiles that share
-    // operand panels), dealt out by descending work in snake order.
-    const int xcd = blockIdx.x % NUM_XCD, pos = blockIdx.x / NUM_XCD;
-    constexpr int SUPER = SUPER_M * SUPER_N;
-    const int round = pos / SUPER, slot = pos % SUPER;
-    const int srank = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - xcd : xcd);
-    if (srank >= n_super) return;
-    const int sid = __builtin_amdgcn_readfirstlane(order[srank]);
-    const int mi = (sid / nSupN) * SUPER_M + slot / SUPER_N, mj = (sid % nSupN) * SUPER_N + slot % SUPER_N;
-    if (mi >= nMacM || mj >= nMacN) return;
-    const int macro = mi * nMacN + mj;
+    // Workgroup b runs on XCD b % NUM_XCD and is that XCD's q-th workgroup,
+    // q = b / NUM_XCD; `order` holds each XCD's sequence: computing macro tiles
+    // (heaviest level first), then the ones with nothing kept.  A computing
+    // workgroup afterwards zero-fills its share of the latter (q + nc,
+    // q + 2 nc, ...), so those stores drain while other workgroups compute.
+    const int xcd = blockIdx.x % NUM_XCD, q = blockIdx.x / NUM_XCD;
+    const int nc = __builtin_amdgcn_readfirstlane(sched[xcd]);
+    const int ntot = __builtin_amdgcn_readfirstlane(sched[NUM_XCD + xcd]);
+    if (q >= ntot || (nc > 0 && q >= nc)) return;
+    SPAMM_TRACE(0);
+    const int32_t *seq = order + (int64_t)xcd * P;
+    const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
+    const int mi = macro / nMacN, mj = macro % nMacN;
     const int U = __builtin_amdgcn_readfirstlane(macro_count[2 * macro]);
     const int Ufull = __builtin_amdgcn_readfirstlane(macro_count[2 * macro + 1]);
     entry_ptr ents = (entry_ptr)(uintptr_t)(macro_list + (int64_t)macro * nbK);
@@ -106,13 +114,16 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
-    if (S == 0) {
-        // nothing kept in this macro tile: C still has to be overwritten with zeros
+    auto zero_fill = [&](int mz) {
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        const int64_t r0 = (int64_t)mi * 256, c0 = (int64_t)mj * 256 + lane * 4;
+        const int64_t r0 = (int64_t)(mz / nMacN) * 256, c0 = (int64_t)(mz % nMacN) * 256 + lane * 4;
         if (c0 < N)
             for (int r = wave; r < 256 && r0 + r < M; r += 4)
                 *reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0) = zero;
+    };
+    if (S == 0) {
+        // nothing kept anywhere on this XCD's list (nc == 0): every workgroup zero-fills its own tile
+        zero_fill(macro);
         return;
     }
 
@@ -219,6 +230,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2) + 2, 0));
         __syncthreads();
 
+        SPAMM_TRACE(1);
         int t = 0;
         // ---- loop 1: entries kept by all tiles of the macro tile; no
         // branches.  Operand vectors are double buffered in registers (a0/b0:
@@ -284,6 +296,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 }
             }
         }
+        SPAMM_TRACE(2);
         // ---- loop 2: entries kept by some tiles only; a wave multiplies
         // exactly the (tile row, tile column) pairs whose bit is set
         for (; t < S; t++) {
@@ -299,9 +312,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                     const int bit = (wr * G::SUB + a) * G::MT + wc * G::SUB + b;
                     sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
                 }
-#ifdef SPAMM_EXP_NOLOOP2
-            sb = 0;
-#endif
             if (sb != 0) {
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++) {
@@ -332,14 +342,12 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 #undef SPAMM_LDA
 #undef SPAMM_LDB
 #undef SPAMM_ISSUE
+        SPAMM_TRACE(3);
         // the ring still holds clamped loads: let them land before the
         // workgroup gives its LDS back
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     }
 
-#ifdef SPAMM_EXP_NOEPI
-    if (acc[0][0][0] != 12345.0f) return;
-#endif
     // ---- epilogue: C[row, col], row-major, ld N (cuSpAMM.cu:391).  MFMA
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
     // column l%32 of the block.
@@ -357,6 +365,19 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         }
     }
 
+
+    // ---- zero-fill this workgroup's share of the macro tiles with nothing kept
+    for (int e = nc + q; e < ntot; e += nc) zero_fill(__builtin_amdgcn_readfirstlane(seq[e]));
+#ifdef SPAMM_EXP_TRACE
+    SPAMM_TRACE(4);
+    if (threadIdx.x == 0) {
+        unsigned hwid, xccid;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xccid));
+        g_trace[(size_t)blockIdx.x * 8 + 5] = ((unsigned long long)xccid << 32) | hwid;
+        g_trace[(size_t)blockIdx.x * 8 + 6] = (unsigned long long)S | ((unsigned long long)Sfull << 32);
+    }
+#endif
 }
 
 static int g_nbuf = 4;
@@ -386,11 +407,8 @@ hipError_t gemm_init() {
 template <int B, int NBUF>
 static void launch_one(unsigned grid, const unsigned char *pA, const unsigned char *pB, const GateBuffers &g,
                        int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C, hipStream_t s) {
-    const int MT = GemmCfg<B>::MT;
-    const int nMacM = (nbM + MT - 1) / MT;
-    const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
     k_gemm<B, NBUF><<<grid, 256, NBUF * GemmCfg<B>::STAGE_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count, g.order,
-                                                                     nSupM * nSupN, nSupN, nMacM, nbM, nbK, nbN,
+                                                                     g.sched, (int)(grid / NUM_XCD), nbM, nbK, nbN,
                                                                      nMacN, M, N, C);
 }
 
@@ -408,8 +426,8 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
-    const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
-    const int rounds = (nSupM * nSupN + NUM_XCD - 1) / NUM_XCD;
+    (void)nMacM;
+    const int rounds = sched_rounds(tile, nbM, nbN);
     const unsigned grid = (unsigned)(rounds * NUM_XCD * SUPER_M * SUPER_N);
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
@@ -421,5 +439,11 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     }
     return hipGetLastError();
 }
+
+#ifdef SPAMM_EXP_TRACE
+extern "C" __attribute__((visibility("default"))) int spamm_debug_trace(void *host, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), bytes);
+}
+#endif
 
 }  // namespace spamm

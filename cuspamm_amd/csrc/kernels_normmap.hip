@@ -38,142 +38,141 @@ __device__ __forceinline__ float butterfly64(float v) {
     return v;
 }
 
-// ------------------------------------------------------------------ role A
-// One wave per tile.  Lane L covers chunk column q = L % (B/8) of rows
-// rl + it*RPI, rl = L / (B/8): every wave-wide load reads RPI full tile rows
-// (B*4 contiguous bytes each) and the chunk index of lane L at step `it` is
-// exactly it*64 + L, so the canonical order needs no data exchange.
-template <int B>
-__global__ __launch_bounds__(256) void k_normmap_a(const float *__restrict__ X, int64_t ld,
-                                                   int64_t nbc, int64_t ntiles,
-                                                   uint4 *__restrict__ packed,
-                                                   float *__restrict__ nm) {
-    constexpr int QN = B / 8;
-    constexpr int RPI = 64 / QN;
-    constexpr int IT = B / RPI;
-    constexpr int UN = IT < 8 ? IT : 8;
-    const int lane = threadIdx.x & 63;
-    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= ntiles) return;
-    const int64_t I = t / nbc, J = t % nbc;
-    const int q = lane % QN, rl = lane / QN;
-    const float *src = X + (I * B + rl) * ld + J * B + 8 * q;
-    uint4 *dst = packed + t * (B * B / 8) + q * B + rl;
-    float partial = 0.0f;
-    for (int it0 = 0; it0 < IT; it0 += UN) {
-        f32x4 v0[UN], v1[UN];
-#pragma unroll
-        for (int u = 0; u < UN; u++) {
-            const f32x4 *p = reinterpret_cast<const f32x4 *>(src + (int64_t)(it0 + u) * RPI * ld);
-            v0[u] = __builtin_nontemporal_load(p);
-            v1[u] = __builtin_nontemporal_load(p + 1);
-        }
-#pragma unroll
-        for (int u = 0; u < UN; u++) {
-            float s = 0.0f;
-            uint4 o;
-            o.x = cvt_pack2(v0[u].x, v0[u].y, s);
-            o.y = cvt_pack2(v0[u].z, v0[u].w, s);
-            o.z = cvt_pack2(v1[u].x, v1[u].y, s);
-            o.w = cvt_pack2(v1[u].z, v1[u].w, s);
-            partial = partial + s;
-            dst[(it0 + u) * RPI] = o;
-        }
-    }
-    partial = butterfly64(partial);
-    if (lane == 0) nm[t] = sqrtf(partial);
-}
-
-// ------------------------------------------------------------------ role B
-// The contraction axis is the row axis, so a lane needs 8 consecutive rows of
-// one column.  Lane L reads a float4 (4 columns) from 8 consecutive rows and
-// transposes in registers: 4 output vectors of 8 halves, 64 contiguous bytes
-// of the packed tile.  A wave covers CW = max(B,64) columns (two tiles when
-// B = 32) and KGPI k-groups per step.  Chunk sums go through a wave-private
-// LDS strip so that the canonical order can be applied afterwards.
-template <int B>
-__global__ __launch_bounds__(256) void k_normmap_b(const float *__restrict__ X, int64_t ld,
-                                                   int64_t nbK, int64_t nbN, int64_t nJw,
-                                                   uint4 *__restrict__ packed,
-                                                   float *__restrict__ nm,
-                                                   float *__restrict__ nmT) {
-    constexpr int CW = B < 64 ? 64 : B;
-    constexpr int TPW = CW / B;           // tiles per wave
-    constexpr int L4 = CW / 4;            // lanes across one row
-    constexpr int KGPI = 64 / L4;         // k-groups per step
+// One workgroup (4 waves) per strip of B rows x 256 columns (256/B tiles).
+//   load    every wave-wide load is one full strip row: 1 KiB contiguous;
+//           wave w takes the 8-row groups w, w+4, ...; all loads of a lane
+//           are in flight together.
+//   convert A role: a lane holds half a chunk (4 of 8 elements along k); the
+//           odd lane continues the even lane's running sum (DPP) so that the
+//           chunk is summed left to right.  B role: a lane holds 8 rows x 4
+//           columns and transposes in registers into 4 k-contiguous vectors.
+//   stage   fp16 vectors go to LDS in the packed tile layout (k-group
+//           segments padded by 16 bytes against bank conflicts), chunk sums
+//           to LDS at their canonical index.
+//   store   after one barrier: the tiles are copied out with contiguous 1 KiB
+//           wave stores (a packed tile is one contiguous block in memory), and
+//           one wave per tile applies the canonical reduction.
+template <int B, int ROLE>
+__global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, int64_t ld, int64_t cols,
+                                                 int64_t nbr, int64_t nbc, int64_t nstrip,
+                                                 uint4 *__restrict__ packed, float *__restrict__ nm,
+                                                 float *__restrict__ nmT) {
+    constexpr int TPS = 256 / B;          // tiles per strip
     constexpr int QN = B / 8;             // k-groups per tile
-    constexpr int IT = QN / KGPI;
-    constexpr int PITCH = QN + 1;         // padded LDS row: conflict-free dump
-    constexpr int STEPS = B * B / 8 / 64;
-    __shared__ float lds[4][TPW * B * PITCH];
+    constexpr int VPT = B * B / 8;        // 16-byte vectors per tile
+    constexpr int QS = B * 16 + 16;       // bytes per k-group segment in LDS (padded)
+    constexpr int TS = QN * QS;           // bytes per tile in LDS
+    constexpr int PITCH = QN + 1;         // padded row of the chunk-sum table
+    constexpr int CH = B * PITCH;         // floats per tile in the chunk-sum table
+    constexpr int NGW = B / 32;           // 8-row groups per wave
+    constexpr int STEPS = VPT / 64;
+    __shared__ __attribute__((aligned(16))) unsigned char s_pack[TPS * TS];
+    __shared__ float s_chunk[TPS * CH];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t w = (int64_t)blockIdx.x * 4 + wave;
-    const bool active = w < nbK * nJw;
-    const int64_t Kt = active ? w / nJw : 0;
-    const int64_t Jw = active ? w % nJw : 0;
-    const int n4 = lane % L4, kgl = lane / L4;
-    const int64_t col0 = Jw * CW + 4 * n4;
-    const bool valid = active && col0 < nbN * B;
-    const int ts = (4 * n4) / B;                 // which tile of the wave
-    const int nl = (4 * n4) % B;                 // first column inside that tile
-    const int64_t J = Jw * TPW + ts;
-    float *strip = lds[wave];
+    const int64_t I = blockIdx.x / nstrip;            // tile row of the strip
+    const int64_t sc = blockIdx.x % nstrip;
+    const int64_t col0 = sc * 256;
+    const int cl = 4 * lane;                          // first column of this lane inside the strip
+    const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
+    const bool valid = col0 + cl < cols;
+    const float *base = X + (I * B) * ld + col0 + cl;
 
-    if (valid) {
-        uint4 *dtile = packed + (J * nbK + Kt) * (int64_t)(B * B / 8);
+    f32x4 v[NGW][8];
 #pragma unroll
-        for (int it = 0; it < IT; it++) {
-            const int kg = it * KGPI + kgl;
-            const float *src = X + (Kt * B + kg * 8) * ld + col0;
-            f32x4 v[8];
+    for (int i = 0; i < NGW; i++)
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                v[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + j * ld));
+        for (int j = 0; j < 8; j++) {
+            const int r = 8 * (wave + 4 * i) + j;
+            if (valid)
+                v[i][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(base + (int64_t)r * ld));
+            else
+                v[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+
+    if (ROLE == 0) {
+        const int q = cin / 8, h = (cin % 8) / 4;
+#pragma unroll
+        for (int i = 0; i < NGW; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int r = 8 * (wave + 4 * i) + j;
+                const _Float16 h0 = (_Float16)v[i][j].x, h1 = (_Float16)v[i][j].y;
+                const _Float16 h2 = (_Float16)v[i][j].z, h3 = (_Float16)v[i][j].w;
+                const float f0 = (float)h0, f1 = (float)h1, f2 = (float)h2, f3 = (float)h3;
+                float s = 0.0f;
+                s = s + f0 * f0; s = s + f1 * f1; s = s + f2 * f2; s = s + f3 * f3;
+                // odd lane: continue from the even neighbour's sum (elements 0..3 of the chunk)
+                const float nb = __builtin_bit_cast(
+                    float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xA0, 0xF, 0xF, false));
+                float s8 = nb;
+                s8 = s8 + f0 * f0; s8 = s8 + f1 * f1; s8 = s8 + f2 * f2; s8 = s8 + f3 * f3;
+                const half2v p0 = {h0, h1}, p1 = {h2, h3};
+                uint2 o;
+                o.x = __builtin_bit_cast(uint32_t, p0);
+                o.y = __builtin_bit_cast(uint32_t, p1);
+                *reinterpret_cast<uint2 *>(s_pack + t * TS + q * QS + r * 16 + h * 8) = o;
+                if (h) s_chunk[t * CH + r * PITCH + q] = s8;
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NGW; i++) {
+            const int kg = wave + 4 * i;
             uint4 o[4];
             float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            o[0].x = cvt_pack2(v[0].x, v[1].x, s[0]);
-            o[0].y = cvt_pack2(v[2].x, v[3].x, s[0]);
-            o[0].z = cvt_pack2(v[4].x, v[5].x, s[0]);
-            o[0].w = cvt_pack2(v[6].x, v[7].x, s[0]);
-            o[1].x = cvt_pack2(v[0].y, v[1].y, s[1]);
-            o[1].y = cvt_pack2(v[2].y, v[3].y, s[1]);
-            o[1].z = cvt_pack2(v[4].y, v[5].y, s[1]);
-            o[1].w = cvt_pack2(v[6].y, v[7].y, s[1]);
-            o[2].x = cvt_pack2(v[0].z, v[1].z, s[2]);
-            o[2].y = cvt_pack2(v[2].z, v[3].z, s[2]);
-            o[2].z = cvt_pack2(v[4].z, v[5].z, s[2]);
-            o[2].w = cvt_pack2(v[6].z, v[7].z, s[2]);
-            o[3].x = cvt_pack2(v[0].w, v[1].w, s[3]);
-            o[3].y = cvt_pack2(v[2].w, v[3].w, s[3]);
-            o[3].z = cvt_pack2(v[4].w, v[5].w, s[3]);
-            o[3].w = cvt_pack2(v[6].w, v[7].w, s[3]);
-            uint4 *d = dtile + kg * B + nl;
+            o[0].x = cvt_pack2(v[i][0].x, v[i][1].x, s[0]);
+            o[0].y = cvt_pack2(v[i][2].x, v[i][3].x, s[0]);
+            o[0].z = cvt_pack2(v[i][4].x, v[i][5].x, s[0]);
+            o[0].w = cvt_pack2(v[i][6].x, v[i][7].x, s[0]);
+            o[1].x = cvt_pack2(v[i][0].y, v[i][1].y, s[1]);
+            o[1].y = cvt_pack2(v[i][2].y, v[i][3].y, s[1]);
+            o[1].z = cvt_pack2(v[i][4].y, v[i][5].y, s[1]);
+            o[1].w = cvt_pack2(v[i][6].y, v[i][7].y, s[1]);
+            o[2].x = cvt_pack2(v[i][0].z, v[i][1].z, s[2]);
+            o[2].y = cvt_pack2(v[i][2].z, v[i][3].z, s[2]);
+            o[2].z = cvt_pack2(v[i][4].z, v[i][5].z, s[2]);
+            o[2].w = cvt_pack2(v[i][6].z, v[i][7].z, s[2]);
+            o[3].x = cvt_pack2(v[i][0].w, v[i][1].w, s[3]);
+            o[3].y = cvt_pack2(v[i][2].w, v[i][3].w, s[3]);
+            o[3].z = cvt_pack2(v[i][4].w, v[i][5].w, s[3]);
+            o[3].w = cvt_pack2(v[i][6].w, v[i][7].w, s[3]);
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                d[c] = o[c];
-                strip[(ts * B + nl + c) * PITCH + kg] = s[c];
+                *reinterpret_cast<uint4 *>(s_pack + t * TS + kg * QS + (cin + c) * 16) = o[c];
+                s_chunk[t * CH + (cin + c) * PITCH + kg] = s[c];
             }
         }
     }
     __syncthreads();
-    if (!active) return;
+
+    // packed tiles out: 256 threads x 16 bytes = 4 KiB per step, contiguous per tile
 #pragma unroll
-    for (int tsel = 0; tsel < TPW; tsel++) {
-        const int64_t Jt = Jw * TPW + tsel;
-        if (Jt >= nbN) break;
+    for (int i = 0; i < TPS * VPT / 256; i++) {
+        const int vi = threadIdx.x + 256 * i;
+        const int tt = vi / VPT, iv = vi % VPT;
+        const int64_t Jt = sc * TPS + tt;
+        if (Jt < nbc) {
+            const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
+            const int64_t tile = ROLE == 0 ? I * nbc + Jt : Jt * nbr + I;
+            packed[tile * VPT + iv] = d;
+        }
+    }
+    // norms: one wave per tile, canonical order
+    for (int tt = wave; tt < TPS; tt += 4) {
+        const int64_t Jt = sc * TPS + tt;
+        if (Jt >= nbc) break;
         float partial = 0.0f;
+#pragma unroll
         for (int it = 0; it < STEPS; it++) {
             const int c = it * 64 + lane;
-            const int r = c / QN, q = c % QN;
-            partial = partial + strip[(tsel * B + r) * PITCH + q];
+            partial = partial + s_chunk[tt * CH + (c / QN) * PITCH + (c % QN)];
         }
         partial = butterfly64(partial);
         if (lane == 0) {
             const float nv = sqrtf(partial);
-            nm[Kt * nbN + Jt] = nv;
-            nmT[Jt * nbK + Kt] = nv;
+            nm[I * nbc + Jt] = nv;
+            if (ROLE == 1) nmT[Jt * nbr + I] = nv;
         }
     }
 }
@@ -247,33 +246,29 @@ __global__ __launch_bounds__(256) void k_fill_decay(float *__restrict__ X, int64
 }
 
 // ---------------------------------------------------------------- launchers
-hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
-                            float *nm, hipStream_t s) {
+template <int ROLE>
+static hipError_t launch_normmap(const float *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
+                                 float *nmT, hipStream_t s) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
-    const int64_t ntiles = nbr * nbc;
-    const unsigned grid = (unsigned)((ntiles + 3) / 4);
+    const int64_t nstrip = (cols + 255) / 256;
+    const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
-        case 32: k_normmap_a<32><<<grid, 256, 0, s>>>(X, cols, nbc, ntiles, (uint4 *)packed, nm); break;
-        case 64: k_normmap_a<64><<<grid, 256, 0, s>>>(X, cols, nbc, ntiles, (uint4 *)packed, nm); break;
-        case 128: k_normmap_a<128><<<grid, 256, 0, s>>>(X, cols, nbc, ntiles, (uint4 *)packed, nm); break;
+        case 32: k_normmap<32, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 64: k_normmap<64, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 128: k_normmap<128, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
+hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+                            float *nm, hipStream_t s) {
+    return launch_normmap<0>(X, rows, cols, tile, packed, nm, nullptr, s);
+}
+
 hipError_t launch_normmap_b(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, float *nmT, hipStream_t s) {
-    const int64_t nbK = rows / tile, nbN = cols / tile;
-    const int cw = tile < 64 ? 64 : tile;
-    const int64_t nJw = (cols + cw - 1) / cw;
-    const unsigned grid = (unsigned)((nbK * nJw + 3) / 4);
-    switch (tile) {
-        case 32: k_normmap_b<32><<<grid, 256, 0, s>>>(X, cols, nbK, nbN, nJw, (uint4 *)packed, nm, nmT); break;
-        case 64: k_normmap_b<64><<<grid, 256, 0, s>>>(X, cols, nbK, nbN, nJw, (uint4 *)packed, nm, nmT); break;
-        case 128: k_normmap_b<128><<<grid, 256, 0, s>>>(X, cols, nbK, nbN, nJw, (uint4 *)packed, nm, nmT); break;
-        default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
+    return launch_normmap<1>(X, rows, cols, tile, packed, nm, nmT, s);
 }
 
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,

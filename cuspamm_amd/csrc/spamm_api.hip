@@ -33,7 +33,7 @@ struct spamm_ctx {
     float tau = 0.0f;
 
     DevBuf packedA, packedB, nA, nB, nBt;
-    DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, kept_total;
+    DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, sched, kept_total;
     DevBuf scratch;   // read-back staging / decay table
 
     hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -95,6 +95,7 @@ GateBuffers gate_buffers(spamm_ctx *c) {
     g.macro_count = (int32_t *)c->macro_count.p;
     g.macro_work = (int32_t *)c->macro_work.p;
     g.order = (int32_t *)c->order.p;
+    g.sched = (int32_t *)c->sched.p;
     g.kept_total = (int64_t *)c->kept_total.p;
     return g;
 }
@@ -168,7 +169,7 @@ int spamm_destroy(spamm_ctx *c) {
     (void)hipStreamSynchronize(c->stream);
     DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->counts, &c->klist,
                       &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
-                      &c->kept_total, &c->scratch};
+                      &c->sched, &c->kept_total, &c->scratch};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     for (int i = 0; i < 5; i++)
@@ -269,7 +270,8 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
     if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
     if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
-    if ((rc = ensure(c, c->order, (size_t)s.n_macro * 4))) return rc;
+    if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * NUM_XCD * SUPER_M * SUPER_N * 2 * 4))) return rc;
+    if ((rc = ensure(c, c->sched, 2 * NUM_XCD * 4))) return rc;
     if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
     HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->stream));

@@ -30,6 +30,15 @@ inline int macro_dim(int tile) { return 256 / tile; }
 constexpr int SUPER_M = 4;
 constexpr int SUPER_N = 8;
 constexpr int NUM_XCD = 8;
+constexpr int SCHED_LEVELS = 16;   // work classes used to order macro tiles inside an XCD
+
+// Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin.
+inline int sched_rounds(int tile, int64_t nbM, int64_t nbN) {
+    const int MT = 256 / tile;
+    const int nMacM = (int)((nbM + MT - 1) / MT), nMacN = (int)((nbN + MT - 1) / MT);
+    const int n_super = ((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N);
+    return (n_super + NUM_XCD - 1) / NUM_XCD;
+}
 
 // One entry of a macro tile's union k list: tile column/row k of the
 // operands plus the set of output tiles (bit a*MT+b = tile row a, column b of
@@ -51,7 +60,8 @@ struct GateBuffers {
     MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
     int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
     int32_t *macro_work;    // [n_macro]       kept products in the macro tile
-    int32_t *order;         // [n_super]       super tiles by descending work
+    int32_t *order;         // [2][8 * P]      macro tile of XCD x's q-th workgroup (P = rounds * 32), -1 = none; second half is scratch
+    int32_t *sched;         // [16]            per XCD: computing items, all items
     int64_t *kept_total;    // [1]  kept products
 };
 
