@@ -38,10 +38,11 @@ __device__ __forceinline__ float butterfly64(float v) {
     return v;
 }
 
-// One workgroup (4 waves) per strip of B rows x 256 columns (256/B tiles).
-//   load    every wave-wide load is one full strip row: 1 KiB contiguous;
-//           wave w takes the 8-row groups w, w+4, ...; all loads of a lane
-//           are in flight together.
+// One workgroup (4 waves) per strip of B rows x SW columns (SW/B tiles; SW =
+// 256, or 128 for B = 128 so that the strip still fits 3 workgroups per CU).
+//   load    every wave-wide load covers 64*4/SW full strip rows, each SW*4
+//           contiguous bytes; a lane takes whole 8-row groups; all loads of a
+//           lane are in flight together.
 //   convert A role: a lane holds half a chunk (4 of 8 elements along k); the
 //           odd lane continues the even lane's running sum (DPP) so that the
 //           chunk is summed left to right.  B role: a lane holds 8 rows x 4
@@ -52,19 +53,21 @@ __device__ __forceinline__ float butterfly64(float v) {
 //   store   after one barrier: the tiles are copied out with contiguous 1 KiB
 //           wave stores (a packed tile is one contiguous block in memory), and
 //           one wave per tile applies the canonical reduction.
-template <int B, int ROLE>
+template <int B, int ROLE, int SW>
 __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT) {
-    constexpr int TPS = 256 / B;          // tiles per strip
+    constexpr int TPS = SW / B;           // tiles per strip
+    constexpr int LPR = SW / 4;           // lanes across one strip row
+    constexpr int RH = 64 / LPR;          // strip rows per wave-wide load
     constexpr int QN = B / 8;             // k-groups per tile
     constexpr int VPT = B * B / 8;        // 16-byte vectors per tile
     constexpr int QS = B * 16 + 16;       // bytes per k-group segment in LDS (padded)
     constexpr int TS = QN * QS;           // bytes per tile in LDS
     constexpr int PITCH = QN + 1;         // padded row of the chunk-sum table
     constexpr int CH = B * PITCH;         // floats per tile in the chunk-sum table
-    constexpr int NGW = B / 32;           // 8-row groups per wave
+    constexpr int NGW = B / (32 * RH);    // 8-row groups per lane
     constexpr int STEPS = VPT / 64;
     __shared__ __attribute__((aligned(16))) unsigned char s_pack[TPS * TS];
     __shared__ float s_chunk[TPS * CH];
@@ -73,8 +76,9 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
     const int wave = threadIdx.x >> 6;
     const int64_t I = blockIdx.x / nstrip;            // tile row of the strip
     const int64_t sc = blockIdx.x % nstrip;
-    const int64_t col0 = sc * 256;
-    const int cl = 4 * lane;                          // first column of this lane inside the strip
+    const int64_t col0 = sc * SW;
+    const int cl = 4 * (lane % LPR);                  // first column of this lane inside the strip
+    const int g0 = wave * RH + lane / LPR;            // first 8-row group of this lane; then every 4*RH-th
     const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
     const bool valid = col0 + cl < cols;
     const float *base = X + (I * B) * ld + col0 + cl;
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
     for (int i = 0; i < NGW; i++)
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const int r = 8 * (wave + 4 * i) + j;
+            const int r = 8 * (g0 + 4 * RH * i) + j;
             if (valid)
                 v[i][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(base + (int64_t)r * ld));
             else
@@ -97,7 +101,7 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
         for (int i = 0; i < NGW; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const int r = 8 * (wave + 4 * i) + j;
+                const int r = 8 * (g0 + 4 * RH * i) + j;
                 const _Float16 h0 = (_Float16)v[i][j].x, h1 = (_Float16)v[i][j].y;
                 const _Float16 h2 = (_Float16)v[i][j].z, h3 = (_Float16)v[i][j].w;
                 const float f0 = (float)h0, f1 = (float)h1, f2 = (float)h2, f3 = (float)h3;
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
     } else {
 #pragma unroll
         for (int i = 0; i < NGW; i++) {
-            const int kg = wave + 4 * i;
+            const int kg = g0 + 4 * RH * i;
             uint4 o[4];
             float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             o[0].x = cvt_pack2(v[i][0].x, v[i][1].x, s[0]);
@@ -250,12 +254,13 @@ template <int ROLE>
 static hipError_t launch_normmap(const float *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
                                  float *nmT, hipStream_t s) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
-    const int64_t nstrip = (cols + 255) / 256;
+    const int sw = tile == 128 ? 128 : 256;
+    const int64_t nstrip = (cols + sw - 1) / sw;
     const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
-        case 32: k_normmap<32, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 64: k_normmap<64, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 128: k_normmap<128, ROLE><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 32: k_normmap<32, ROLE, 256><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 64: k_normmap<64, ROLE, 256><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 128: k_normmap<128, ROLE, 128><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
