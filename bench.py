@@ -27,6 +27,14 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
+# HBM bytes per launch for the headline workload, from rocprofv3 --pmc FETCH_SIZE and --pmc
+# WRITE_SIZE runs of this file (KiB per dispatch; summaries and scale factors under profiles/).
+# They describe the committed kernels and are None for other workloads.
+MEASURED_TRAFFIC = {
+    # fetch counter x 2.0 (a plain 1 GiB copy reads 524303 KiB on FETCH_SIZE), write counter x 1.0
+    "headline": {"gemm": 4.0725e9, "normmap": 1.6114e9},
+}
+
 WORKLOADS = {
     # name: (N, tile, kind, lam, target kept ratio or None, fixed tau or None)
     "headline": (16384, 64, "exp", 0.003, 0.10, None),
@@ -46,17 +54,6 @@ def decay_table(kind, n, lam):
     else:
         t = np.ones(n)
     return np.ascontiguousarray(t, dtype=np.float32)
-
-
-def tau_for_ratio(nA, nB, ratio):
-    """Exact order statistic over the fp32 norm products (host, outside the timed region)."""
-    p = (nA[:, None, :] * nB.T[None, :, :]).reshape(-1)
-    want = max(1, int(np.ceil(ratio * p.size)))
-    tau = np.partition(p, p.size - want)[p.size - want]
-    if not tau > 0:
-        pos = p[p > 0]
-        tau = pos.min() if pos.size else np.float32(0)
-    return float(tau), float((p >= tau).mean())
 
 
 def cpu_baseline(A, B, tile, tau, budget_s):
@@ -113,6 +110,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-literal", action="store_true", help="skip the one-off run of the literal lam=0.1 config")
     ap.add_argument("--cpu-budget", type=float, default=12.0, help="seconds of host GEMM in the CPU sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build is single-GPU by design (the SpAMM path runs on one MI355X); "
@@ -125,6 +124,15 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
 
+    if args.calibrate_copy:
+        x = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        y = torch.empty_like(x)
+        for _ in range(5):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": x.numel() * 4, "bytes_written": x.numel() * 4, "launches": 5}))
+        return
+
     N, tile, kind, lam, ratio, tau = WORKLOADS[args.workload]
     nb = N // tile
     ctx = sp.SpammContext(0)          # runs on torch's current stream
@@ -136,9 +144,10 @@ def main():
     dC = torch.empty((N, N), dtype=torch.float32, device="cuda")
 
     if tau is None:
+        # fixed before the timed region: exact order statistic over the norm products, on the device
         ctx.normmap_f32(sp.ROLE_B, dB, tile)
         ctx.normmap_f32(sp.ROLE_A, dA, tile)
-        tau, achieved = tau_for_ratio(ctx.get_normmap(sp.ROLE_A), ctx.get_normmap(sp.ROLE_B), ratio)
+        tau, achieved = ctx.tau_for_ratio(ratio)
     else:
         achieved = None
 
@@ -195,16 +204,30 @@ def main():
         "roofline": {
             "kernel": "k_gemm<%d> (gated MFMA GEMM)" % tile, "bound": "mfma",
             "achieved": round(gemm_tflops, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gemm_tflops / PEAK_FP16_TFLOPS, 4), "traffic": None,
+            "frac": round(gemm_tflops / PEAK_FP16_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("gemm"),
             "flops_per_launch": flops, "avg_launch_ms": round(stage[3], 4),
         },
         "roofline_normmap": {
             "kernel": "k_normmap_a/b<%d> (fp32->fp16 + tile norms)" % tile, "bound": "hbm",
             "achieved": round(nm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(nm_gbs / PEAK_HBM_GBS, 4), "traffic": None,
+            "frac": round(nm_gbs / PEAK_HBM_GBS, 4),
+            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("normmap"),
             "bytes_per_launch": nm_bytes, "avg_launch_ms": round((stage[0] + stage[1]) / 2, 4),
         },
     }
+
+    # error against an exact fp64 dense product of the same fp16 operands, whole matrix, next to
+    # the tau-derived bound (both formed on the device, outside the timed region)
+    if N <= 16384:
+        ctx.multiply(dA, dB, tile, tau, C=dC)
+        e64, d64, c64 = ctx.error_vs_dense(dC)
+        out["error_vs_fp64_dense"] = {
+            "frobenius_error": float("%.6e" % e64), "dense_frobenius": float("%.6e" % d64),
+            "relative": float("%.3e" % (e64 / d64 if d64 else 0.0)),
+            "tau_bound_frobenius": float("%.6e" % ctx.dropped_bound(tau)),
+            "rows": N,
+        }
 
     if args.workload == "headline" and not args.skip_literal:
         # the decay rate as literally written in the config, run once for the record
@@ -215,7 +238,7 @@ def main():
         ctx.fill_decay(lB, tab_l, 2)
         ctx.normmap_f32(sp.ROLE_B, lB, tile)
         ctx.normmap_f32(sp.ROLE_A, lA, tile)
-        ltau, lach = tau_for_ratio(ctx.get_normmap(sp.ROLE_A), ctx.get_normmap(sp.ROLE_B), 0.10)
+        ltau, lach = ctx.tau_for_ratio(0.10)
         best = 1e9
         for _ in range(5):
             ctx.multiply(lA, lB, tile, ltau, C=dC, timing=True)

@@ -14,5 +14,7 @@ from .api import (  # noqa: F401
     SpammParams,
     SpammStats,
     load_library,
+    load_csv,
+    load_mtx,
     library_path,
 )

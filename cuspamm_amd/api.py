@@ -15,6 +15,8 @@ ROLE_A = 0
 ROLE_B = 1
 FLAG_A_EQ_B = 1
 FLAG_TIMING = 2
+FLAG_REUSE_A = 4
+FLAG_REUSE_B = 8
 
 OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV = 0, -1, -2, -3, -4, -5
 
@@ -66,9 +68,21 @@ def load_library():
     L.spamm_set_stream.argtypes = [vp, vp]
     L.spamm_multiply.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
     L.spamm_normmap_f32.argtypes = [vp, ctypes.c_int, vp, i64, i64, i32]
+    L.spamm_normmap_f16.argtypes = [vp, ctypes.c_int, vp, i64, i64, i32]
+    L.spamm_multiply_f16.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
+    L.spamm_error_vs_dense_f64.argtypes = [vp, vp, i64, i64, ctypes.POINTER(ctypes.c_double)]
+    L.spamm_dropped_bound.argtypes = [vp, f32, ctypes.POINTER(ctypes.c_double)]
+    L.spamm_load_csv_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
+    L.spamm_load_mtx_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
     L.spamm_gate.argtypes = [vp, f32]
     L.spamm_gemm_gated.argtypes = [vp, vp]
     L.spamm_set_normmaps.argtypes = [vp, vp, vp, i64, i64, i64, i32]
+    L.spamm_tau_for_ratio.argtypes = [vp, ctypes.c_double, ctypes.POINTER(ctypes.c_float),
+                                      ctypes.POINTER(ctypes.c_double)]
+    L.spamm_tune_bisect.argtypes = [vp, ctypes.c_double, ctypes.c_double, ctypes.c_int,
+                                    ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    L.spamm_count_kept.argtypes = [vp, ctypes.c_double, ctypes.POINTER(ctypes.c_int64),
+                                   ctypes.POINTER(ctypes.c_double)]
     L.spamm_get_normmap.argtypes = [vp, ctypes.c_int, vp]
     L.spamm_get_counts.argtypes = [vp, vp]
     L.spamm_get_klist.argtypes = [vp, vp]
@@ -150,7 +164,10 @@ class SpammContext:
         return int(self._lib.spamm_last_hip_error(self._h))
 
     # -- the multiply call
-    def multiply(self, A, B, tile, tau, C=None, timing=False):
+    def multiply(self, A, B, tile, tau, C=None, timing=False, reuse_a=False, reuse_b=False):
+        """C = SpAMM(A, B).  fp32 or fp16 inputs (both the same dtype).  With reuse_a / reuse_b the
+        operand's fp16 copy and norm map from the previous call are kept (pass the same tensor, it
+        only supplies the shape)."""
         import torch
         if A.dim() != 2 or B.dim() != 2:
             raise ValueError("A and B must be matrices")
@@ -158,12 +175,20 @@ class SpammContext:
         K2, N = B.shape
         if K != K2:
             raise ValueError("inner dimensions differ")
+        if A.dtype != B.dtype:
+            raise TypeError("A and B must have the same dtype")
         if C is None:
             C = torch.empty((M, N), dtype=torch.float32, device=A.device)
-        p = SpammParams(M, K, N, int(tile), float(tau), FLAG_TIMING if timing else 0, 0)
-        _check(self._lib.spamm_multiply(self._h, ctypes.byref(p), _devptr(A, "float32"),
-                                        _devptr(B, "float32"), _devptr(C, "float32")),
-               "spamm_multiply")
+        flags = (FLAG_TIMING if timing else 0) | (FLAG_REUSE_A if reuse_a else 0) | (FLAG_REUSE_B if reuse_b else 0)
+        p = SpammParams(M, K, N, int(tile), float(tau), flags, 0)
+        if A.dtype == torch.float16:
+            _check(self._lib.spamm_multiply_f16(self._h, ctypes.byref(p), _devptr(A, "float16"),
+                                                _devptr(B, "float16"), _devptr(C, "float32")),
+                   "spamm_multiply_f16")
+        else:
+            _check(self._lib.spamm_multiply(self._h, ctypes.byref(p), _devptr(A, "float32"),
+                                            _devptr(B, "float32"), _devptr(C, "float32")),
+                   "spamm_multiply")
         self._shape = (M // tile, K // tile, N // tile, int(tile), M, K, N)
         return C
 
@@ -184,6 +209,32 @@ class SpammContext:
             s[1], s[2], s[5], s[6] = rows // tile, cols // tile, rows, cols
         self._shape = tuple(s)
 
+    def normmap_f16(self, role, X, tile):
+        rows, cols = X.shape
+        _check(self._lib.spamm_normmap_f16(self._h, int(role), _devptr(X, "float16"), rows, cols,
+                                           int(tile)), "spamm_normmap_f16")
+        s = list(self._shape) if self._shape and self._shape[3] == tile else [0, 0, 0, tile, 0, 0, 0]
+        if role == ROLE_A:
+            s[0], s[1], s[4], s[5] = rows // tile, cols // tile, rows, cols
+        else:
+            s[1], s[2], s[5], s[6] = rows // tile, cols // tile, rows, cols
+        self._shape = tuple(s)
+
+    def error_vs_dense(self, C, row0=0, row1=None):
+        """(||C - D||_F, ||D||_F, ||C||_F) over rows [row0, row1), D = exact fp64 product of the
+        resident fp16 operands."""
+        if row1 is None:
+            row1 = C.shape[0]
+        out = (ctypes.c_double * 3)()
+        _check(self._lib.spamm_error_vs_dense_f64(self._h, _devptr(C, "float32"), int(row0), int(row1), out),
+               "spamm_error_vs_dense_f64")
+        return out[0], out[1], out[2]
+
+    def dropped_bound(self, tau):
+        out = ctypes.c_double(0)
+        _check(self._lib.spamm_dropped_bound(self._h, float(tau), ctypes.byref(out)), "spamm_dropped_bound")
+        return float(out.value)
+
     def set_normmaps(self, nA, nB, tile):
         nA = np.ascontiguousarray(nA, dtype=np.float32)
         nB = np.ascontiguousarray(nB, dtype=np.float32)
@@ -197,6 +248,25 @@ class SpammContext:
 
     def gate(self, tau):
         _check(self._lib.spamm_gate(self._h, float(tau)), "spamm_gate")
+
+    # -- tau selection (norm maps must be present)
+    def tau_for_ratio(self, ratio):
+        tau, ach = ctypes.c_float(0), ctypes.c_double(0)
+        _check(self._lib.spamm_tau_for_ratio(self._h, float(ratio), ctypes.byref(tau), ctypes.byref(ach)),
+               "spamm_tau_for_ratio")
+        return float(tau.value), float(ach.value)
+
+    def tune_bisect(self, expected=0.75, tol=0.01, max_rounds=20):
+        tau, ach = ctypes.c_float(0), ctypes.c_double(0)
+        _check(self._lib.spamm_tune_bisect(self._h, float(expected), float(tol), int(max_rounds),
+                                           ctypes.byref(tau), ctypes.byref(ach)), "spamm_tune_bisect")
+        return float(tau.value), float(ach.value)
+
+    def count_kept(self, threshold):
+        cnt, sm = ctypes.c_int64(0), ctypes.c_double(0)
+        _check(self._lib.spamm_count_kept(self._h, float(threshold), ctypes.byref(cnt), ctypes.byref(sm)),
+               "spamm_count_kept")
+        return int(cnt.value), float(sm.value)
 
     def gemm_gated(self, C):
         _check(self._lib.spamm_gemm_gated(self._h, _devptr(C, "float32")), "spamm_gemm_gated")
@@ -250,3 +320,19 @@ class SpammContext:
                                               table.ctypes.data, int(seed), 1 if random else 0),
                "spamm_fill_decay_f32")
         return X
+
+
+def load_csv(path, rows, cols, ld=None):
+    """Dense CSV, one matrix row per line, into a zero-filled (rows, ld) fp32 array (host)."""
+    ld = cols if ld is None else ld
+    out = np.empty((rows, ld), dtype=np.float32)
+    _check(load_library().spamm_load_csv_f32(os.fsencode(path), rows, cols, ld, out.ctypes.data), "spamm_load_csv_f32")
+    return out
+
+
+def load_mtx(path, rows, cols, ld=None):
+    """'row col val' triples (1-based, first line skipped) into a zero-filled (rows, ld) fp32 array (host)."""
+    ld = cols if ld is None else ld
+    out = np.empty((rows, ld), dtype=np.float32)
+    _check(load_library().spamm_load_mtx_f32(os.fsencode(path), rows, cols, ld, out.ctypes.data), "spamm_load_mtx_f32")
+    return out

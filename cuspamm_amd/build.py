@@ -12,7 +12,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libspamm_gfx950.so")
 
-SOURCES = ["kernels_normmap.hip", "kernels_gate.hip", "kernels_gemm.hip", "spamm_api.hip"]
+SOURCES = ["kernels_normmap.hip", "kernels_gate.hip", "kernels_gemm.hip", "kernels_tau.hip", "kernels_tools.hip",
+           "spamm_api.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 

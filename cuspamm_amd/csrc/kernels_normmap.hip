@@ -53,8 +53,8 @@ __device__ __forceinline__ float butterfly64(float v) {
 //   store   after one barrier: the tiles are copied out with contiguous 1 KiB
 //           wave stores (a packed tile is one contiguous block in memory), and
 //           one wave per tile applies the canonical reduction.
-template <int B, int ROLE, int SW>
-__global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, int64_t ld, int64_t cols,
+template <int B, int ROLE, int SW, bool IN16>
+__global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT) {
@@ -81,7 +81,9 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
     const int g0 = wave * RH + lane / LPR;            // first 8-row group of this lane; then every 4*RH-th
     const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
     const bool valid = col0 + cl < cols;
-    const float *base = X + (I * B) * ld + col0 + cl;
+    // IN16: the input already is fp16 (the reference's own input type, para.h:1); the
+    // conversion below is then the identity and only the packing and the norms remain
+    const int64_t eoff = (I * B) * ld + col0 + cl;
 
     f32x4 v[NGW][8];
 #pragma unroll
@@ -89,10 +91,17 @@ __global__ __launch_bounds__(256) void k_normmap(const float *__restrict__ X, in
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int r = 8 * (g0 + 4 * RH * i) + j;
-            if (valid)
-                v[i][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(base + (int64_t)r * ld));
-            else
+            if (!valid) {
                 v[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            } else if (IN16) {
+                typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+                const half4v hv = __builtin_nontemporal_load(
+                    reinterpret_cast<const half4v *>(static_cast<const _Float16 *>(Xv) + eoff + (int64_t)r * ld));
+                v[i][j] = f32x4{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+            } else {
+                v[i][j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const f32x4 *>(static_cast<const float *>(Xv) + eoff + (int64_t)r * ld));
+            }
         }
 
     if (ROLE == 0) {
@@ -250,30 +259,32 @@ __global__ __launch_bounds__(256) void k_fill_decay(float *__restrict__ X, int64
 }
 
 // ---------------------------------------------------------------- launchers
-template <int ROLE>
-static hipError_t launch_normmap(const float *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
+template <int ROLE, bool IN16>
+static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
                                  float *nmT, hipStream_t s) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
     const int sw = tile == 128 ? 128 : 256;
     const int64_t nstrip = (cols + sw - 1) / sw;
     const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
-        case 32: k_normmap<32, ROLE, 256><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 64: k_normmap<64, ROLE, 256><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 128: k_normmap<128, ROLE, 128><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+hipError_t launch_normmap_a(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, hipStream_t s) {
-    return launch_normmap<0>(X, rows, cols, tile, packed, nm, nullptr, s);
+    return in16 ? launch_normmap<0, true>(X, rows, cols, tile, packed, nm, nullptr, s)
+                : launch_normmap<0, false>(X, rows, cols, tile, packed, nm, nullptr, s);
 }
 
-hipError_t launch_normmap_b(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, float *nmT, hipStream_t s) {
-    return launch_normmap<1>(X, rows, cols, tile, packed, nm, nmT, s);
+    return in16 ? launch_normmap<1, true>(X, rows, cols, tile, packed, nm, nmT, s)
+                : launch_normmap<1, false>(X, rows, cols, tile, packed, nm, nmT, s);
 }
 
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,

@@ -3,7 +3,10 @@
 // (TGPUplan, cuSpAMM.cu:6-12, 433-451).  See include/spamm.h for the contract.
 #include "../../include/spamm.h"
 
+#include <math.h>
 #include <new>
+#include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <vector>
 
@@ -35,6 +38,7 @@ struct spamm_ctx {
     DevBuf packedA, packedB, nA, nB, nBt;
     DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, sched, kept_total;
     DevBuf scratch;   // read-back staging / decay table
+    DevBuf tauws;     // tau selection workspace
 
     hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     bool timing = false;        // events of the last multiply are valid
@@ -169,7 +173,7 @@ int spamm_destroy(spamm_ctx *c) {
     (void)hipStreamSynchronize(c->stream);
     DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->counts, &c->klist,
                       &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
-                      &c->sched, &c->kept_total, &c->scratch};
+                      &c->sched, &c->kept_total, &c->scratch, &c->tauws};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     for (int i = 0; i < 5; i++)
@@ -193,8 +197,8 @@ int spamm_synchronize(spamm_ctx *c) {
     return SPAMM_OK;
 }
 
-int spamm_normmap_f32(spamm_ctx *c, int role, const float *dX, int64_t rows, int64_t cols,
-                      int32_t tile) {
+static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_t rows, int64_t cols,
+                       int32_t tile) {
     if (!c || !dX || !tile_ok(tile)) return SPAMM_EINVAL;
     if (role != SPAMM_ROLE_A && role != SPAMM_ROLE_B) return SPAMM_EINVAL;
     if (rows <= 0 || cols <= 0 || rows % tile || cols % tile) return SPAMM_EINVAL;
@@ -211,7 +215,7 @@ int spamm_normmap_f32(spamm_ctx *c, int role, const float *dX, int64_t rows, int
         if ((rc = ensure(c, c->packedA, (size_t)rows * cols * 2))) return rc;
         if ((rc = ensure(c, c->nA, nt * 4))) return rc;
         if (c->timing) HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
-        HIPCHK(c, launch_normmap_a(dX, rows, cols, tile, c->packedA.p, (float *)c->nA.p, c->stream));
+        HIPCHK(c, launch_normmap_a(dX, in16, rows, cols, tile, c->packedA.p, (float *)c->nA.p, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[2], c->stream)); c->ev_a = true; }
         c->have_a = true;
     } else {
@@ -222,13 +226,23 @@ int spamm_normmap_f32(spamm_ctx *c, int role, const float *dX, int64_t rows, int
         if ((rc = ensure(c, c->nB, nt * 4))) return rc;
         if ((rc = ensure(c, c->nBt, nt * 4))) return rc;
         if (c->timing) HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
-        HIPCHK(c, launch_normmap_b(dX, rows, cols, tile, c->packedB.p, (float *)c->nB.p,
+        HIPCHK(c, launch_normmap_b(dX, in16, rows, cols, tile, c->packedB.p, (float *)c->nB.p,
                                    (float *)c->nBt.p, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[1], c->stream)); c->ev_b = true; }
         c->have_b = true;
     }
     c->have_gate = false;
     return SPAMM_OK;
+}
+
+int spamm_normmap_f32(spamm_ctx *c, int role, const float *dX, int64_t rows, int64_t cols,
+                      int32_t tile) {
+    return normmap_any(c, role, dX, false, rows, cols, tile);
+}
+
+int spamm_normmap_f16(spamm_ctx *c, int role, const void *dXh, int64_t rows, int64_t cols,
+                      int32_t tile) {
+    return normmap_any(c, role, dXh, true, rows, cols, tile);
 }
 
 int spamm_set_normmaps(spamm_ctx *c, const float *nA, const float *nB, int64_t nbM, int64_t nbK,
@@ -293,9 +307,11 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     return SPAMM_OK;
 }
 
-int spamm_multiply(spamm_ctx *c, const spamm_params *p, const float *dA, const float *dB,
-                   float *dC) {
-    if (!c || !p || !dA || !dB || !dC) return SPAMM_EINVAL;
+static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, const void *dB, bool in16,
+                        float *dC) {
+    if (!c || !p || !dC) return SPAMM_EINVAL;
+    const bool reuse_a = (p->flags & SPAMM_FLAG_REUSE_A) != 0, reuse_b = (p->flags & SPAMM_FLAG_REUSE_B) != 0;
+    if ((!dA && !reuse_a) || (!dB && !reuse_b)) return SPAMM_EINVAL;
     if (!tile_ok(p->tile)) return SPAMM_EINVAL;
     if (p->M <= 0 || p->K <= 0 || p->N <= 0) return SPAMM_EINVAL;
     if (p->M % p->tile || p->K % p->tile || p->N % p->tile) return SPAMM_EINVAL;
@@ -304,10 +320,221 @@ int spamm_multiply(spamm_ctx *c, const spamm_params *p, const float *dA, const f
     c->ev_a = c->ev_b = c->ev_gate = c->ev_gemm = false;
     int rc;
     // same order as the reference: B's norm map first, then A's (cuSpAMM.cu:478-503)
-    if ((rc = spamm_normmap_f32(c, SPAMM_ROLE_B, dB, p->K, p->N, p->tile))) return rc;
-    if ((rc = spamm_normmap_f32(c, SPAMM_ROLE_A, dA, p->M, p->K, p->tile))) return rc;
+    // an operand flagged for reuse must be resident with the same shape and tile
+    if (reuse_a && !(c->have_a && c->tile == p->tile && c->M == p->M && c->K == p->K)) return SPAMM_ESTATE;
+    if (reuse_b && !(c->have_b && c->tile == p->tile && c->K == p->K && c->N == p->N)) return SPAMM_ESTATE;
+    if (!reuse_b) {
+        if ((rc = normmap_any(c, SPAMM_ROLE_B, dB, in16, p->K, p->N, p->tile))) return rc;
+    } else if (c->timing) {
+        HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
+        HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
+        c->ev_b = true;
+    }
+    if (!reuse_a) {
+        if ((rc = normmap_any(c, SPAMM_ROLE_A, dA, in16, p->M, p->K, p->tile))) return rc;
+    } else if (c->timing) {
+        HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
+        c->ev_a = true;
+    }
     if ((rc = spamm_gate(c, p->tau))) return rc;
     if ((rc = spamm_gemm_gated(c, dC))) return rc;
+    return SPAMM_OK;
+}
+
+int spamm_multiply(spamm_ctx *c, const spamm_params *p, const float *dA, const float *dB, float *dC) {
+    return multiply_any(c, p, dA, dB, false, dC);
+}
+
+int spamm_multiply_f16(spamm_ctx *c, const spamm_params *p, const void *dAh, const void *dBh, float *dC) {
+    return multiply_any(c, p, dAh, dBh, true, dC);
+}
+
+int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_t row1, double *out3) {
+    if (!c || !dC || !out3) return SPAMM_EINVAL;
+    if (!c->have_a || !c->have_b) return SPAMM_ESTATE;
+    if (row0 < 0 || row1 > c->M || row0 >= row1 || row0 % 64 || row1 % 64 || c->N % 64 || c->K % 16)
+        return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    if ((rc = ensure(c, c->tauws, tau_workspace_bytes()))) return rc;
+    double *d = (double *)c->tauws.p;
+    HIPCHK(c, launch_error_vs_dense(c->packedA.p, c->packedB.p, c->M, c->K, c->N, c->tile, dC, row0, row1, d,
+                                    c->stream));
+    double sq[3];
+    if ((rc = copy_out(c, d, sq, sizeof(sq)))) return rc;
+    for (int i = 0; i < 3; i++) out3[i] = sqrt(sq[i]);
+    return SPAMM_OK;
+}
+
+int spamm_dropped_bound(spamm_ctx *c, float tau, double *out) {
+    if (!c || !out || tau != tau) return SPAMM_EINVAL;
+    Shape s;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    int rc = set_device(c);
+    if (rc) return rc;
+    s = shape_of(c);
+    if ((rc = ensure(c, c->tauws, tau_workspace_bytes()))) return rc;
+    double *d = (double *)c->tauws.p;
+    HIPCHK(c, launch_dropped_bound((const float *)c->nA.p, (const float *)c->nBt.p, s.nbM, s.nbK, s.nbN, tau, d,
+                                   c->stream));
+    double sq;
+    if ((rc = copy_out(c, d, &sq, sizeof(sq)))) return rc;
+    *out = sqrt(sq);
+    return SPAMM_OK;
+}
+
+// ---- input adapters (host side; getMatrixFromCSV / getMatrixFromMTX, tool.cu:282-366)
+static int load_text(const char *path, std::vector<char> &buf) {
+    FILE *f = fopen(path, "rb");
+    if (!f) return SPAMM_EINVAL;
+    fseek(f, 0, SEEK_END);
+    long n = ftell(f);
+    fseek(f, 0, SEEK_SET);
+    if (n < 0) { fclose(f); return SPAMM_EINVAL; }
+    buf.resize((size_t)n + 1);
+    size_t got = fread(buf.data(), 1, (size_t)n, f);
+    fclose(f);
+    buf[got] = 0;
+    return SPAMM_OK;
+}
+
+int spamm_load_csv_f32(const char *path, int64_t rows, int64_t cols, int64_t ld, float *host_out) {
+    if (!path || !host_out || rows <= 0 || cols <= 0 || ld < cols) return SPAMM_EINVAL;
+    std::vector<char> buf;
+    int rc = load_text(path, buf);
+    if (rc) return rc;
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < ld; j++) host_out[i * ld + j] = 0.0f;
+    char *p = buf.data();
+    for (int64_t i = 0; i < rows && *p; i++) {            // one line per matrix row, at most `rows` lines
+        char *eol = strchr(p, '\n');
+        if (eol) *eol = 0;
+        int64_t j = 0;
+        char *q = p;
+        while (*q && j < cols) {
+            char *end;
+            float x = strtof(q, &end);
+            if (end == q) x = 0.0f;                       // empty / unparsable field reads as 0
+            host_out[i * ld + j++] = x;
+            char *comma = strchr(q, ',');
+            if (!comma) break;
+            q = comma + 1;
+        }
+        if (!eol) break;
+        p = eol + 1;
+    }
+    return SPAMM_OK;
+}
+
+int spamm_load_mtx_f32(const char *path, int64_t rows, int64_t cols, int64_t ld, float *host_out) {
+    if (!path || !host_out || rows <= 0 || cols <= 0 || ld < cols) return SPAMM_EINVAL;
+    std::vector<char> buf;
+    int rc = load_text(path, buf);
+    if (rc) return rc;
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < ld; j++) host_out[i * ld + j] = 0.0f;
+    char *p = buf.data();
+    bool first = true;
+    while (*p) {
+        char *eol = strchr(p, '\n');
+        if (eol) *eol = 0;
+        if (first) {
+            first = false;                                // the first line (header / sizes) is skipped
+        } else {
+            long long r, cidx;
+            double v;
+            if (sscanf(p, "%lld %lld %lf", &r, &cidx, &v) == 3) {   // 1-based "row col val"
+                if (r < 1 || r > rows || cidx < 1 || cidx > cols) return SPAMM_EINVAL;
+                host_out[(r - 1) * ld + (cidx - 1)] = (float)v;
+            }
+        }
+        if (!eol) break;
+        p = eol + 1;
+    }
+    return SPAMM_OK;
+}
+
+static int tau_prepare(spamm_ctx *c, Shape *s) {
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    int rc = set_device(c);
+    if (rc) return rc;
+    *s = shape_of(c);
+    return ensure(c, c->tauws, tau_workspace_bytes());
+}
+
+static int tau_count(spamm_ctx *c, const Shape &s, double thr, TauCounts *out) {
+    HIPCHK(c, launch_tau_count((const float *)c->nA.p, (const float *)c->nBt.p, s.nbM, s.nbK, s.nbN, thr,
+                               c->tauws.p, c->stream));
+    return copy_out(c, (char *)c->tauws.p + tau_counts_offset(), out, sizeof(*out));
+}
+
+int spamm_count_kept(spamm_ctx *c, double threshold, int64_t *count_out, double *sum_out) {
+    if (!c || threshold != threshold) return SPAMM_EINVAL;
+    Shape s;
+    int rc = tau_prepare(c, &s);
+    if (rc) return rc;
+    TauCounts tc;
+    if ((rc = tau_count(c, s, threshold, &tc))) return rc;
+    if (count_out) *count_out = (int64_t)tc.count;
+    if (sum_out) *sum_out = tc.sum;
+    return SPAMM_OK;
+}
+
+int spamm_tau_for_ratio(spamm_ctx *c, double ratio, float *tau_out, double *achieved_out) {
+    if (!c || !tau_out || !(ratio >= 0.0) || ratio > 1.0) return SPAMM_EINVAL;
+    Shape s;
+    int rc = tau_prepare(c, &s);
+    if (rc) return rc;
+    const unsigned long long total = (unsigned long long)s.nbM * s.nbK * s.nbN;
+    TauCounts tc;
+    if ((rc = tau_count(c, s, 0.0, &tc))) return rc;
+    double w = ceil(ratio * (double)total);
+    unsigned long long want = w < 1.0 ? 1ull : (unsigned long long)w;
+    if (want > total) want = total;
+    if (tc.positive == 0) {                 // nothing but zeros: only tau = 0 keeps anything
+        *tau_out = 0.0f;
+        if (achieved_out) *achieved_out = 1.0;
+        return SPAMM_OK;
+    }
+    if (want > tc.positive) want = tc.positive;     // zero tail: settle for the smallest positive product
+    HIPCHK(c, launch_tau_select((const float *)c->nA.p, (const float *)c->nBt.p, s.nbM, s.nbK, s.nbN, want,
+                                c->tauws.p, c->stream));
+    TauState st;
+    if ((rc = copy_out(c, c->tauws.p, &st, sizeof(st)))) return rc;
+    memcpy(tau_out, &st.tau_bits, 4);
+    if (achieved_out) *achieved_out = (double)st.kept / (double)total;
+    return SPAMM_OK;
+}
+
+int spamm_tune_bisect(spamm_ctx *c, double expected, double tol, int max_rounds, float *tau_out,
+                      double *achieved_out) {
+    if (!c || !tau_out || max_rounds < 1 || !(tol > 0.0)) return SPAMM_EINVAL;
+    Shape s;
+    int rc = tau_prepare(c, &s);
+    if (rc) return rc;
+    const long long total = (long long)(s.nbM * s.nbK * s.nbN);
+    double Norm = 0, up = 0, down = 0, rate = 0;
+    for (int Ti = 0; Ti < max_rounds; Ti++) {       // tool.cu:445-486
+        TauCounts tc;
+        if ((rc = tau_count(c, s, Norm, &tc))) return rc;
+        rate = (double)((float)tc.count / (float)total);
+        if (fabs(rate - expected) < tol) break;
+        if (Ti == 0) {
+            Norm = tc.sum / (double)total;
+            up = Norm;
+            continue;
+        }
+        if (rate > expected) {
+            if (up == Norm) up *= 2;
+            down = Norm;
+            Norm = (Norm + up) / 2;
+        } else {
+            up = Norm;
+            Norm = (Norm + down) / 2;
+        }
+    }
+    *tau_out = (float)Norm;
+    if (achieved_out) *achieved_out = rate;
     return SPAMM_OK;
 }
 

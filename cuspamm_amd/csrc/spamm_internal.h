@@ -65,10 +65,16 @@ struct GateBuffers {
     int64_t *kept_total;    // [1]  kept products
 };
 
-hipError_t launch_normmap_a(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+hipError_t launch_normmap_a(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, hipStream_t s);
-hipError_t launch_normmap_b(const float *X, int64_t rows, int64_t cols, int tile, void *packed,
+hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, float *nmT, hipStream_t s);
+// error report tooling (kernels_tools.hip)
+hipError_t launch_error_vs_dense(const void *packedA, const void *packedB, int64_t M, int64_t K, int64_t N,
+                                 int tile, const float *C, int64_t row0, int64_t row1, double *out3,
+                                 hipStream_t s);
+hipError_t launch_dropped_bound(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
+                                float tau, double *out1, hipStream_t s);
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,
                          uint16_t *out, hipStream_t s);
 hipError_t launch_transpose_normmap(const float *nB, int64_t nbK, int64_t nbN, float *nBt,
@@ -79,6 +85,26 @@ hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *
 size_t gate_lds_bytes(int tile, int64_t nbK);
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
                        float tau, hipStream_t s);
+
+// tau selection (kernels_tau.hip)
+struct TauState {
+    unsigned long long want;      // rank (1-based, from the top) still to find inside the prefix
+    unsigned long long greater;   // products strictly above the current prefix range
+    unsigned long long kept;      // products >= tau (valid after the last pass)
+    uint32_t prefix;              // decided high bits, right-aligned
+    uint32_t tau_bits;
+};
+struct TauCounts {
+    unsigned long long count;     // products with (double)p >= threshold
+    unsigned long long positive;  // products > 0
+    double sum;                   // sum of all products
+};
+size_t tau_workspace_bytes();
+inline size_t tau_counts_offset() { return 64 + 2048 * 8; }
+hipError_t launch_tau_select(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
+                             unsigned long long want, void *workspace, hipStream_t s);
+hipError_t launch_tau_count(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
+                            double thr, void *workspace, hipStream_t s);
 
 hipError_t gemm_init();   // one-time kernel attribute set-up
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,

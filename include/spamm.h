@@ -42,6 +42,8 @@ extern "C" {
 /* spamm_params.flags */
 #define SPAMM_FLAG_A_EQ_B 1u     /* A and B are the same matrix (square); reserved */
 #define SPAMM_FLAG_TIMING 2u     /* record per-stage HIP events (spamm_get_stats) */
+#define SPAMM_FLAG_REUSE_A 4u    /* A's fp16 copy and norm map from an earlier call are reused (dA ignored) */
+#define SPAMM_FLAG_REUSE_B 8u    /* same for B: e.g. one B against many A, or matrix powers */
 
 /* Run-time form of the reference's compile-time configuration:
  * M,K,N <- inM,inK,inN (para.h:6-8) already padded to a tile multiple
@@ -88,12 +90,21 @@ SPAMM_API int spamm_set_stream(spamm_ctx *ctx, void *hip_stream);
 SPAMM_API int spamm_multiply(spamm_ctx *ctx, const spamm_params *p, const float *dA, const float *dB,
                    float *dC);
 
+/* The same multiply for operands that already are fp16 (the reference's actual
+ * input type, para.h:1, cuSpAMM.cu:486): dAh, dBh are row-major fp16 device
+ * arrays.  The norm-map stage then only packs and takes norms. */
+SPAMM_API int spamm_multiply_f16(spamm_ctx *ctx, const spamm_params *p, const void *dAh, const void *dBh,
+                                 float *dC);
+
 /* Stage 1 -- replaces unroll_get_Fnorm_FP16 / unroll_get_Fnorm_pri
  * (cuSpAMM.cu:74-123, 21-71; launches :478-503) plus the host fp16 conversion:
  * reads fp32 dX [rows x cols], stores the fp16 copy (context-private packed
  * layout) and the tile Frobenius norm map [rows/tile x cols/tile]. */
 SPAMM_API int spamm_normmap_f32(spamm_ctx *ctx, int role, const float *dX, int64_t rows, int64_t cols,
                       int32_t tile);
+
+SPAMM_API int spamm_normmap_f16(spamm_ctx *ctx, int role, const void *dXh, int64_t rows, int64_t cols,
+                                int32_t tile);
 
 /* Stage 2 -- replaces the gating prologue of get_C_FP16_B32
  * (cuSpAMM.cu:302-334): per output tile the kept-k bitmap, the ascending
@@ -104,6 +115,25 @@ SPAMM_API int spamm_gate(spamm_ctx *ctx, float tau);
 /* Stage 3 -- replaces the product loop of get_C_FP16_B32 (cuSpAMM.cu:336-391):
  * C_ij = sum over kept k of A_ik * B_kj, fp16 operands, fp32 accumulate. */
 SPAMM_API int spamm_gemm_gated(spamm_ctx *ctx, float *dC);
+
+/* tau for a target kept ratio -- replaces the host-side tuner that the reference
+ * runs inside its timed loop (tuneValidRate, tool.cu:438-490; main.h:35-38).
+ * Both use the norm maps left by stage 1 (or spamm_set_normmaps) and leave
+ * the gate untouched.
+ *   spamm_tau_for_ratio: exact order statistic on the device: tau = the
+ *     ceil(ratio*total)-th largest fp32 norm product, so that the products
+ *     >= tau are kept (ties may push the achieved ratio above the target); if
+ *     fewer positive products exist, the smallest positive one.
+ *   spamm_tune_bisect: the reference's bisection, same arithmetic
+ *     (tool.cu:445-486): round 0 measures the ratio at tau = 0 and moves to the
+ *     mean product, later rounds bisect, stop at |ratio - expected| < tol or
+ *     after max_rounds (reference: 0.75, 0.01, 20).  Counting runs on the device.
+ *   spamm_count_kept: products with (double)product >= threshold, and the
+ *     sum of all products (tool.cu:448-463, 505-516). */
+SPAMM_API int spamm_tau_for_ratio(spamm_ctx *ctx, double ratio, float *tau_out, double *achieved_out);
+SPAMM_API int spamm_tune_bisect(spamm_ctx *ctx, double expected, double tol, int max_rounds, float *tau_out,
+                                double *achieved_out);
+SPAMM_API int spamm_count_kept(spamm_ctx *ctx, double threshold, int64_t *count_out, double *sum_out);
 
 /* Upload host norm maps (row-major nA [nbM x nbK], nB [nbK x nbN]) so that the
  * gate can be exercised on hand-built maps. */
@@ -132,6 +162,22 @@ SPAMM_API int spamm_get_stats(spamm_ctx *ctx, spamm_stats *out);
  * random == 0.  `table` is a HOST array of max(rows,cols) floats. */
 SPAMM_API int spamm_fill_decay_f32(spamm_ctx *ctx, float *dX, int64_t rows, int64_t cols,
                          const float *host_table, uint64_t seed, int random);
+
+/* Error report (check_simple_gpu / COUNTERRTRANS, tool.cu:227-280, 6-24, with an
+ * exact fp64 product of the resident fp16 operands instead of cuBLAS):
+ * out3 = { ||C - C_dense||_F, ||C_dense||_F, ||C||_F } over rows [row0, row1)
+ * (multiples of 64; N a multiple of 64).  The dense product is never stored. */
+SPAMM_API int spamm_error_vs_dense_f64(spamm_ctx *ctx, const float *dC, int64_t row0, int64_t row1,
+                                       double *out3);
+/* tau-derived bound on that error: sqrt(sum_ij (sum_{k dropped} nA[i,k]*nB[k,j])^2). */
+SPAMM_API int spamm_dropped_bound(spamm_ctx *ctx, float tau, double *out);
+
+/* Input adapters (host): dense CSV, one matrix row per line (getMatrixFromCSV,
+ * tool.cu:329-366), and "row col val" triples, 1-based, first line skipped
+ * (getMatrixFromMTX, tool.cu:282-327).  host_out is rows x ld, zero-filled
+ * first, so ld/rows may be the tile-padded sizes (main.h:54-56). */
+SPAMM_API int spamm_load_csv_f32(const char *path, int64_t rows, int64_t cols, int64_t ld, float *host_out);
+SPAMM_API int spamm_load_mtx_f32(const char *path, int64_t rows, int64_t cols, int64_t ld, float *host_out);
 
 SPAMM_API int spamm_synchronize(spamm_ctx *ctx);
 SPAMM_API const char *spamm_strerror(int code);

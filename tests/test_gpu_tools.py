@@ -1,0 +1,77 @@
+"""fp16-input entry point, operand reuse and the error-report tooling."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+@pytest.mark.parametrize("tile", [32, 64, 128])
+def test_fp16_inputs_equal_fp32_inputs_of_the_same_values(orc, ctx, tile):
+    import torch
+    M, K, N = 3 * 128, 2 * 128, 4 * 128
+    tab = orc.decay_table("exp", max(M, K, N), 0.01)
+    A = _dev(orc.fill_decay(M, K, tab, 1)).half()
+    B = _dev(orc.fill_decay(K, N, tab, 2)).half()
+    ctx.normmap_f16(1, B, tile)
+    ctx.normmap_f16(0, A, tile)
+    tau, ach = ctx.tau_for_ratio(0.5)
+    assert 0.45 < ach < 0.6
+    C16 = ctx.multiply(A, B, tile, tau).clone()
+    m16, nA16, nB16 = ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1)
+    assert np.array_equal(ctx.get_fp16(0), A.cpu().numpy().view(np.uint16))
+    assert np.array_equal(ctx.get_fp16(1), B.cpu().numpy().view(np.uint16))
+    C32 = ctx.multiply(A.float(), B.float(), tile, tau)
+    assert np.array_equal(ctx.get_mask(), m16)
+    assert np.array_equal(ctx.get_normmap(0).view(np.uint32), nA16.view(np.uint32))
+    assert np.array_equal(ctx.get_normmap(1).view(np.uint32), nB16.view(np.uint32))
+    assert torch.equal(C16, C32)
+    kept = ctx.get_stats().kept_products
+    assert 0 < kept < (M // tile) * (K // tile) * (N // tile)
+
+
+def test_operand_reuse(orc, ctx):
+    import torch
+    import cuspamm_amd as sp
+    n = 512
+    tab = orc.decay_table("exp", n, 0.01)
+    A1, A2, B = (_dev(orc.fill_decay(n, n, tab, s)) for s in (1, 3, 2))
+    ref1 = ctx.multiply(A1, B, 64, 0.5).clone()
+    ref2 = ctx.multiply(A2, B, 64, 0.5).clone()
+    ctx.multiply(A1, B, 64, 0.5)
+    got2 = ctx.multiply(A2, B, 64, 0.5, reuse_b=True)          # B's fp16 copy and norm map are kept
+    assert torch.equal(got2, ref2)
+    got1 = ctx.multiply(A1, B, 64, 0.5, reuse_b=True)
+    assert torch.equal(got1, ref1)
+    got1 = ctx.multiply(A1, B, 64, 0.1, reuse_a=True, reuse_b=True)   # only tau changes
+    assert torch.equal(got1, ctx.multiply(A1, B, 64, 0.1))
+    with pytest.raises(sp.SpammError) as ei:                    # shape changed: nothing to reuse
+        ctx.multiply(A1[:256].contiguous(), B, 64, 0.5, reuse_a=True)
+    assert ei.value.code == -4
+
+
+def test_error_report_matches_checker(orc, ctx):
+    n, tile = 512, 64
+    tab = orc.decay_table("exp", n, 0.01)
+    A, B = orc.fill_decay(n, n, tab, 1), orc.fill_decay(n, n, tab, 2)
+    for tau in (0.0, 0.5, 3.0):
+        C = ctx.multiply(_dev(A), _dev(B), tile, tau)
+        Af = orc.f16_bits_to_f32(ctx.get_fp16(0))
+        Bf = orc.f16_bits_to_f32(ctx.get_fp16(1))
+        dense = orc.gemm_dense_f64(Af, Bf)
+        e, d, c = orc.frob_diff(C.cpu().numpy(), dense)
+        ge, gd, gc = ctx.error_vs_dense(C)
+        assert abs(gd - d) <= 1e-10 * d and abs(gc - c) <= 1e-10 * c
+        assert abs(ge - e) <= 1e-6 * e + 1e-12 * d
+        bound = orc.dropped_bound(ctx.get_normmap(0), ctx.get_normmap(1), tau)
+        gb = ctx.dropped_bound(tau)
+        assert abs(gb - bound) <= 1e-9 * max(bound, 1e-30)
+        assert ge <= gb * (1 + 1e-4) + 1e-5 * gd
+        # row range
+        ge2, gd2, _ = ctx.error_vs_dense(C, 128, 256)
+        e2, d2, _ = orc.frob_diff(C.cpu().numpy()[128:256], dense[128:256])
+        assert abs(gd2 - d2) <= 1e-10 * d2 and abs(ge2 - e2) <= 1e-6 * e2 + 1e-12 * d2
