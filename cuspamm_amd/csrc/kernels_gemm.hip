@@ -248,7 +248,10 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             load_frags(a0, b0, 0, 0);
             uint32_t knext = stage_k(NBUF);
             for (; t < Sfull; t++) {
-                const uint32_t kissue = knext;
+                // address of the stage issued after this iteration's sync, computed early so that
+                // only the scalar load of the next k sits between the barrier and the MFMAs
+                const StageAddr sa_new = stage_addr(t + NBUF, knext);
+                SPAMM_FENCE();
                 {
                     const unsigned char *bufA = smem + (t % NBUF) * G::STAGE_BYTES;
                     const unsigned char *bufB = bufA + G::A_BYTES;
@@ -277,7 +280,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 SPAMM_FENCE();
                 // scalar load placed here so that no LDS wait follows it closely
                 knext = stage_k(t + 1 + NBUF);
-                sa_tail = stage_addr(t + NBUF, kissue);
+                sa_tail = sa_new;
                 SPAMM_FENCE();
                 {
                     const unsigned char *bufA = smem + ((t + 1) % NBUF) * G::STAGE_BYTES;
@@ -350,7 +353,9 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 
     // ---- epilogue: C[row, col], row-major, ld N (cuSpAMM.cu:391).  MFMA
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
-    // column l%32 of the block.
+    // column l%32 of the block: every store instruction writes two full
+    // 128-byte row segments.  (Swapping the MFMA operands would give float4
+    // stores, but each then touches 32 rows with 32 bytes -- measured slower.)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const int64_t row0 = (int64_t)mi * 256 + wr * 128 + r * 32;
@@ -364,7 +369,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             for (int i = 0; i < 16; i++) out[(int64_t)(8 * (i / 4) + (i % 4)) * N] = acc[r][c][i];
         }
     }
-
 
     // ---- zero-fill this workgroup's share of the macro tiles with nothing kept
     for (int e = nc + q; e < ntot; e += nc) zero_fill(__builtin_amdgcn_readfirstlane(seq[e]));
