@@ -42,6 +42,20 @@ def _run(cmd):
     return out
 
 
+def _check_no_scratch(log, src):
+    """The GEMM keeps 256 accumulator registers per lane; a compiler version or an edit that
+    makes it spill them to scratch memory costs a factor of several, so refuse such a build."""
+    import re
+    name = None
+    for line in log.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and "k_gemm" in name and int(m.group(1)) != 0:
+            raise RuntimeError("%s: kernel %s spills %s bytes/lane to scratch" % (src, name, m.group(1)))
+
+
 def build_library(verbose=False):
     """Compiles every HIP source and links the shared library. Always rebuilds."""
     objdir = os.path.join(CSRC, "build")
@@ -50,7 +64,21 @@ def build_library(verbose=False):
 
     def compile_one(pair):
         src, obj = pair
-        return _run([HIPCC] + CFLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        extra = ["-Rpass-analysis=kernel-resource-usage"] if src == "kernels_gemm.hip" else []
+        log = _run([HIPCC] + CFLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
+        if extra:
+            _check_no_scratch(log, src)
+            keep, skip = [], 0
+            for line in log.splitlines():          # drop the remarks and the source excerpts printed under them
+                if "remark:" in line:
+                    skip = 2
+                elif skip and (line.lstrip().startswith("|") or "|" in line[:8]):
+                    skip -= 1
+                else:
+                    skip = 0
+                    keep.append(line)
+            log = "\n".join(keep)
+        return log
 
     with ThreadPoolExecutor(max_workers=4) as ex:
         logs = list(ex.map(compile_one, zip(SOURCES, objs)))
