@@ -1,0 +1,95 @@
+"""Shape sweep: ragged tile counts, extreme aspect ratios, long k, special values."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+C_REL_TOL = 1e-3
+
+
+def _dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def _check(orc, ctx, A, B, tile, tau):
+    import torch
+    M, N = A.shape[0], B.shape[1]
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ctx.multiply(_dev(A), _dev(B), tile, tau, C=C)
+    ref = orc.spamm(A, B, tile, tau)
+    assert np.array_equal(ctx.get_mask(), ref["mask"])
+    assert np.array_equal(ctx.get_counts(), ref["counts"])
+    assert ctx.get_stats().kept_products == ref["kept"]
+    Cg = C.cpu().numpy()
+    err, nrm, _ = orc.frob_diff(Cg, ref["C"])
+    assert err <= C_REL_TOL * nrm or (nrm == 0 and err == 0)
+    return ref
+
+
+def test_random_shapes(orc, ctx):
+    rng = np.random.default_rng(2024)
+    for trial in range(40):
+        tile = int(rng.choice([32, 64, 128]))
+        M, K, N = (int(rng.integers(1, 1 + 1024 // tile)) * tile for _ in range(3))
+        lam = float(rng.choice([0.0, 0.005, 0.02, 0.1]))
+        tab = orc.decay_table("exp", max(M, K, N), lam)
+        A = orc.fill_decay(M, K, tab, 10 + trial)
+        B = orc.fill_decay(K, N, tab, 100 + trial)
+        nA = orc.normmap(orc.f32_to_f16_bits(A), tile, 0)
+        nB = orc.normmap(orc.f32_to_f16_bits(B), tile, 1)
+        ratio = float(rng.choice([0.0, 0.1, 0.5, 0.9, 1.0]))
+        tau = 0.0 if ratio == 1.0 else (np.inf if ratio == 0.0 else orc.tau_for_ratio(nA, nB, ratio)[0])
+        _check(orc, ctx, A, B, tile, tau)
+
+
+@pytest.mark.parametrize("M,K,N,tile", [(64, 64, 8192, 64), (8192, 64, 64, 64), (64, 16384, 64, 32),
+                                        (128, 32768, 128, 128), (2560, 256, 2304, 64), (32, 32, 32, 32),
+                                        (288, 32, 2080, 32)])
+def test_extreme_aspect_ratios(orc, ctx, M, K, N, tile):
+    tab = orc.decay_table("exp", max(M, K, N), 0.002)
+    A = orc.fill_decay(M, K, tab, 1)
+    B = orc.fill_decay(K, N, tab, 2)
+    nA = orc.normmap(orc.f32_to_f16_bits(A), tile, 0)
+    nB = orc.normmap(orc.f32_to_f16_bits(B), tile, 1)
+    tau, _ = orc.tau_for_ratio(nA, nB, 0.4)
+    ref = _check(orc, ctx, A, B, tile, tau)
+    assert 0 < ref["kept"]
+
+
+def test_scattered_sparsity_pattern(orc, ctx):
+    # no band structure at all: random tiles zeroed, so k lists are ragged and macro tiles mixed
+    rng = np.random.default_rng(7)
+    n, tile = 1024, 64
+    A = rng.uniform(-1, 1, size=(n, n)).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(n, n)).astype(np.float32)
+    za = rng.random((n // tile, n // tile)) < 0.6
+    zb = rng.random((n // tile, n // tile)) < 0.6
+    A *= np.kron(~za, np.ones((tile, tile), dtype=np.float32))
+    B *= np.kron(~zb, np.ones((tile, tile), dtype=np.float32))
+    scale = 10.0 ** rng.integers(-3, 1, size=(n // tile, n // tile))
+    A *= np.kron(scale, np.ones((tile, tile))).astype(np.float32)
+    ref = _check(orc, ctx, A, B, tile, 1.0)
+    assert 0 < ref["kept"] < (n // tile) ** 3 // 2
+
+
+def test_non_finite_inputs_follow_ieee_compare(orc, ctx):
+    # inf tile norm: kept against any non-zero tile; NaN product (inf*0, NaN norm) is dropped
+    n, tile = 256, 64
+    rng = np.random.default_rng(3)
+    A = rng.uniform(-1, 1, size=(n, n)).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(n, n)).astype(np.float32)
+    A[5, 70] = 1e6            # overflows fp16 -> inf in tile (0,1)
+    A[130, 200] = np.nan      # NaN in tile (2,3)
+    B[64:128, 0:64] = 0       # zero tile (1,0): inf * 0 = NaN -> dropped
+    import torch
+    C = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    ctx.multiply(_dev(A), _dev(B), tile, 0.5, C=C)
+    ref = orc.spamm(A, B, tile, 0.5)
+    assert np.array_equal(ctx.get_mask(), ref["mask"])
+    assert np.array_equal(ctx.get_counts(), ref["counts"])
+    Cg, Cr = C.cpu().numpy(), ref["C"]
+    assert np.array_equal(np.isnan(Cg), np.isnan(Cr))
+    assert np.array_equal(np.isinf(Cg), np.isinf(Cr))
+    fin = np.isfinite(Cr)
+    assert np.linalg.norm(Cg[fin] - Cr[fin]) <= C_REL_TOL * np.linalg.norm(Cr[fin])
+    assert not ref["mask"][0, 0, 0] & np.uint64(2)      # (i=0, j=0, k=1): inf * 0 is not kept
