@@ -30,7 +30,7 @@ inline int macro_dim(int tile) { return 256 / tile; }
 constexpr int SUPER_M = 4;
 constexpr int SUPER_N = 8;
 constexpr int NUM_XCD = 8;
-constexpr int SCHED_LEVELS = 16;   // work classes used to order macro tiles inside an XCD
+constexpr int SCHED_LEVELS = 4;   // work classes used to order macro tiles inside an XCD (0 = nothing kept)
 
 // Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin.
 inline int sched_rounds(int tile, int64_t nbM, int64_t nbN) {
