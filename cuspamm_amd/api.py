@@ -164,7 +164,7 @@ class SpammContext:
         return int(self._lib.spamm_last_hip_error(self._h))
 
     # -- the multiply call
-    def multiply(self, A, B, tile, tau, C=None, timing=False, reuse_a=False, reuse_b=False):
+    def multiply(self, A, B, tile, tau, C=None, timing=False, reuse_a=False, reuse_b=False, a_eq_b=False):
         """C = SpAMM(A, B).  fp32 or fp16 inputs (both the same dtype).  With reuse_a / reuse_b the
         operand's fp16 copy and norm map from the previous call are kept (pass the same tensor, it
         only supplies the shape)."""
@@ -179,7 +179,8 @@ class SpammContext:
             raise TypeError("A and B must have the same dtype")
         if C is None:
             C = torch.empty((M, N), dtype=torch.float32, device=A.device)
-        flags = (FLAG_TIMING if timing else 0) | (FLAG_REUSE_A if reuse_a else 0) | (FLAG_REUSE_B if reuse_b else 0)
+        flags = ((FLAG_TIMING if timing else 0) | (FLAG_REUSE_A if reuse_a else 0) |
+                 (FLAG_REUSE_B if reuse_b else 0) | (FLAG_A_EQ_B if a_eq_b else 0))
         p = SpammParams(M, K, N, int(tile), float(tau), flags, 0)
         if A.dtype == torch.float16:
             _check(self._lib.spamm_multiply_f16(self._h, ctypes.byref(p), _devptr(A, "float16"),

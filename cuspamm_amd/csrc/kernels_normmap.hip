@@ -57,7 +57,8 @@ template <int B, int ROLE, int SW, bool IN16>
 __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
-                                                 float *__restrict__ nmT) {
+                                                 float *__restrict__ nmT, uint4 *__restrict__ packed2,
+                                                 float *__restrict__ nm2) {
     constexpr int TPS = SW / B;           // tiles per strip
     constexpr int LPR = SW / 4;           // lanes across one strip row
     constexpr int RH = 64 / LPR;          // strip rows per wave-wide load
@@ -104,7 +105,9 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             }
         }
 
-    if (ROLE == 0) {
+    // ROLE 2 = the same matrix is both operands (A = B): one read of X, both packed layouts and
+    // both norm maps (A role first -> packed/nm, then B role -> packed2/nm2/nmT), LDS reused.
+    auto stage_a = [&]() {
         const int q = cin / 8, h = (cin % 8) / 4;
 #pragma unroll
         for (int i = 0; i < NGW; i++)
@@ -128,7 +131,8 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
                 *reinterpret_cast<uint2 *>(s_pack + t * TS + q * QS + r * 16 + h * 8) = o;
                 if (h) s_chunk[t * CH + r * PITCH + q] = s8;
             }
-    } else {
+    };
+    auto stage_b = [&]() {
 #pragma unroll
         for (int i = 0; i < NGW; i++) {
             const int kg = g0 + 4 * RH * i;
@@ -156,37 +160,54 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
                 s_chunk[t * CH + (cin + c) * PITCH + kg] = s[c];
             }
         }
-    }
-    __syncthreads();
-
-    // packed tiles out: 256 threads x 16 bytes = 4 KiB per step, contiguous per tile
+    };
+    // packed tiles out (256 threads x 16 bytes = 4 KiB per step, contiguous per tile) and norms
+    // (one wave per tile, canonical order)
+    auto emit = [&](bool as_b, uint4 *__restrict__ pk, float *__restrict__ nmo, float *__restrict__ nmTo) {
 #pragma unroll
-    for (int i = 0; i < TPS * VPT / 256; i++) {
-        const int vi = threadIdx.x + 256 * i;
-        const int tt = vi / VPT, iv = vi % VPT;
-        const int64_t Jt = sc * TPS + tt;
-        if (Jt < nbc) {
-            const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
-            const int64_t tile = ROLE == 0 ? I * nbc + Jt : Jt * nbr + I;
-            packed[tile * VPT + iv] = d;
+        for (int i = 0; i < TPS * VPT / 256; i++) {
+            const int vi = threadIdx.x + 256 * i;
+            const int tt = vi / VPT, iv = vi % VPT;
+            const int64_t Jt = sc * TPS + tt;
+            if (Jt < nbc) {
+                const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
+                const int64_t tile = as_b ? Jt * nbr + I : I * nbc + Jt;
+                pk[tile * VPT + iv] = d;
+            }
         }
-    }
-    // norms: one wave per tile, canonical order
-    for (int tt = wave; tt < TPS; tt += 4) {
-        const int64_t Jt = sc * TPS + tt;
-        if (Jt >= nbc) break;
-        float partial = 0.0f;
+        for (int tt = wave; tt < TPS; tt += 4) {
+            const int64_t Jt = sc * TPS + tt;
+            if (Jt >= nbc) break;
+            float partial = 0.0f;
 #pragma unroll
-        for (int it = 0; it < STEPS; it++) {
-            const int c = it * 64 + lane;
-            partial = partial + s_chunk[tt * CH + (c / QN) * PITCH + (c % QN)];
+            for (int it = 0; it < STEPS; it++) {
+                const int c = it * 64 + lane;
+                partial = partial + s_chunk[tt * CH + (c / QN) * PITCH + (c % QN)];
+            }
+            partial = butterfly64(partial);
+            if (lane == 0) {
+                const float nv = sqrtf(partial);
+                nmo[I * nbc + Jt] = nv;
+                if (as_b) nmTo[Jt * nbr + I] = nv;
+            }
         }
-        partial = butterfly64(partial);
-        if (lane == 0) {
-            const float nv = sqrtf(partial);
-            nm[I * nbc + Jt] = nv;
-            if (ROLE == 1) nmT[Jt * nbr + I] = nv;
-        }
+    };
+    if (ROLE == 0) {
+        stage_a();
+        __syncthreads();
+        emit(false, packed, nm, nullptr);
+    } else if (ROLE == 1) {
+        stage_b();
+        __syncthreads();
+        emit(true, packed, nm, nmT);
+    } else {
+        stage_a();
+        __syncthreads();
+        emit(false, packed, nm, nullptr);
+        __syncthreads();
+        stage_b();
+        __syncthreads();
+        emit(true, packed2, nm2, nmT);
     }
 }
 
@@ -261,15 +282,15 @@ __global__ __launch_bounds__(256) void k_fill_decay(float *__restrict__ X, int64
 // ---------------------------------------------------------------- launchers
 template <int ROLE, bool IN16>
 static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
-                                 float *nmT, hipStream_t s) {
+                                 float *nmT, hipStream_t s, void *packed2 = nullptr, float *nm2 = nullptr) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
     const int sw = tile == 128 ? 128 : 256;
     const int64_t nstrip = (cols + sw - 1) / sw;
     const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
-        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
-        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT); break;
+        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
+        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
+        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -279,6 +300,12 @@ hipError_t launch_normmap_a(const void *X, bool in16, int64_t rows, int64_t cols
                             float *nm, hipStream_t s) {
     return in16 ? launch_normmap<0, true>(X, rows, cols, tile, packed, nm, nullptr, s)
                 : launch_normmap<0, false>(X, rows, cols, tile, packed, nm, nullptr, s);
+}
+
+hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void *packedA, float *nmA,
+                             void *packedB, float *nmB, float *nmBt, hipStream_t s) {
+    return in16 ? launch_normmap<2, true>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB)
+                : launch_normmap<2, false>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB);
 }
 
 hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,

@@ -157,12 +157,16 @@ int spamm_create(spamm_ctx **out, int device) {
     if (!c) return SPAMM_ENOMEM;
     c->device = device;
     int rc = set_device(c);
-    if (rc != SPAMM_OK) { delete c; return rc; }
-    if (hipStreamCreate(&c->own_stream) != hipSuccess) { delete c; return SPAMM_EHIP; }
+    if (rc == SPAMM_OK && hipStreamCreate(&c->own_stream) != hipSuccess) rc = SPAMM_EHIP;
     c->stream = c->own_stream;
-    for (int i = 0; i < 5; i++)
-        if (hipEventCreate(&c->ev[i]) != hipSuccess) { delete c; return SPAMM_EHIP; }
-    if (gemm_init() != hipSuccess) { delete c; return SPAMM_EHIP; }
+    for (int i = 0; i < 5 && rc == SPAMM_OK; i++)
+        if (hipEventCreate(&c->ev[i]) != hipSuccess) rc = SPAMM_EHIP;
+    if (rc == SPAMM_OK && gemm_init() != hipSuccess) rc = SPAMM_EHIP;
+    if (rc != SPAMM_OK) {
+        (void)hipGetLastError();
+        spamm_destroy(c);          // releases whatever was created
+        return rc;
+    }
     *out = c;
     return SPAMM_OK;
 }
@@ -170,7 +174,7 @@ int spamm_create(spamm_ctx **out, int device) {
 int spamm_destroy(spamm_ctx *c) {
     if (!c) return SPAMM_EINVAL;
     (void)hipSetDevice(c->device);
-    (void)hipStreamSynchronize(c->stream);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
     DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->counts, &c->klist,
                       &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
                       &c->sched, &c->kept_total, &c->scratch, &c->tauws};
@@ -323,14 +327,42 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     // an operand flagged for reuse must be resident with the same shape and tile
     if (reuse_a && !(c->have_a && c->tile == p->tile && c->M == p->M && c->K == p->K)) return SPAMM_ESTATE;
     if (reuse_b && !(c->have_b && c->tile == p->tile && c->K == p->K && c->N == p->N)) return SPAMM_ESTATE;
-    if (!reuse_b) {
+    const bool a_eq_b = (p->flags & SPAMM_FLAG_A_EQ_B) != 0;
+    if (a_eq_b) {
+        // one read of the matrix feeds both operand roles (the reference's A = B runs convert and
+        // norm the same data twice)
+        if (reuse_a || reuse_b || dA != dB || p->M != p->K || p->K != p->N) return SPAMM_EINVAL;
+        if (c->tile != p->tile) reset_shape(c, p->tile);
+        const int64_t n = p->M;
+        if (n / p->tile > 65535) return SPAMM_EINVAL;
+        if ((rc = set_device(c))) return rc;
+        const size_t nt = (size_t)(n / p->tile) * (size_t)(n / p->tile);
+        if ((rc = ensure(c, c->packedA, (size_t)n * n * 2))) return rc;
+        if ((rc = ensure(c, c->packedB, (size_t)n * n * 2))) return rc;
+        if ((rc = ensure(c, c->nA, nt * 4))) return rc;
+        if ((rc = ensure(c, c->nB, nt * 4))) return rc;
+        if ((rc = ensure(c, c->nBt, nt * 4))) return rc;
+        c->M = c->K = c->N = n;
+        if (c->timing) HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
+        HIPCHK(c, launch_normmap_ab(dA, in16, n, p->tile, c->packedA.p, (float *)c->nA.p, c->packedB.p,
+                                    (float *)c->nB.p, (float *)c->nBt.p, c->stream));
+        if (c->timing) {
+            HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
+            HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
+            c->ev_a = c->ev_b = true;
+        }
+        c->have_a = c->have_b = true;
+        c->have_gate = false;
+    } else if (!reuse_b) {
         if ((rc = normmap_any(c, SPAMM_ROLE_B, dB, in16, p->K, p->N, p->tile))) return rc;
     } else if (c->timing) {
         HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
         HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
         c->ev_b = true;
     }
-    if (!reuse_a) {
+    if (a_eq_b) {
+        // done above
+    } else if (!reuse_a) {
         if ((rc = normmap_any(c, SPAMM_ROLE_A, dA, in16, p->M, p->K, p->tile))) return rc;
     } else if (c->timing) {
         HIPCHK(c, hipEventRecord(c->ev[2], c->stream));

@@ -75,3 +75,26 @@ def test_error_report_matches_checker(orc, ctx):
         ge2, gd2, _ = ctx.error_vs_dense(C, 128, 256)
         e2, d2, _ = orc.frob_diff(C.cpu().numpy()[128:256], dense[128:256])
         assert abs(gd2 - d2) <= 1e-10 * d2 and abs(ge2 - e2) <= 1e-6 * e2 + 1e-12 * d2
+
+
+@pytest.mark.parametrize("tile", [32, 64, 128])
+def test_a_equals_b_single_pass(orc, ctx, tile):
+    # BASELINE config 1 shape (A = B): one read of the matrix must give the same fp16 copies, norm
+    # maps, mask and C as the two-pass run
+    import torch
+    import cuspamm_amd as sp
+    n = 1024
+    tab = orc.decay_table("exp", n, 0.5 if tile == 32 else 0.02)
+    X = _dev(orc.fill_decay(n, n, tab, 1))
+    tau = 1e-4 if tile == 32 else 2.0
+    C2 = ctx.multiply(X, X, tile, tau).clone()
+    ref = (ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1), ctx.get_fp16(0), ctx.get_fp16(1))
+    C1 = ctx.multiply(X, X, tile, tau, a_eq_b=True)
+    got = (ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1), ctx.get_fp16(0), ctx.get_fp16(1))
+    for r, g in zip(ref, got):
+        assert np.array_equal(r.view(np.uint8), g.view(np.uint8))
+    assert torch.equal(C1, C2)
+    kept = ctx.get_stats().kept_products
+    assert 0 < kept < (n // tile) ** 3
+    with pytest.raises(sp.SpammError):                       # the flag needs the same pointer and a square problem
+        ctx.multiply(X, X.clone(), tile, tau, a_eq_b=True)
