@@ -109,6 +109,7 @@ def main():
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-literal", action="store_true", help="skip the one-off run of the literal lam=0.1 config")
+    ap.add_argument("--skip-dense", action="store_true", help="skip the dense fp16 GEMM comparison")
     ap.add_argument("--cpu-budget", type=float, default=12.0, help="seconds of host GEMM in the CPU sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE/WRITE_SIZE)")
@@ -216,6 +217,36 @@ def main():
             "bytes_per_launch": nm_bytes, "avg_launch_ms": round((stage[0] + stage[1]) / 2, 4),
         },
     }
+
+    # what the matrix pipeline sustains on this box with nothing but MFMAs: with random operands
+    # the clock settles well below the datasheet's (power management), so this, not the datasheet
+    # peak, is what a GEMM on real data can approach; and a dense fp16 GEMM of the same size by the
+    # vendor library (the analogue of the reference's cuBLAS comparison, tool.cu:153-226)
+    tf_rand, ghz_rand = ctx.mfma_ceiling(True)
+    tf_zero, ghz_zero = ctx.mfma_ceiling(False)
+    out["mfma_ceiling"] = {
+        "random_operands_tflops": round(tf_rand, 1), "random_operands_clock_ghz": round(ghz_rand, 3),
+        "zero_operands_tflops": round(tf_zero, 1), "zero_operands_clock_ghz": round(ghz_zero, 3),
+        "gemm_frac_of_random_operand_ceiling": round(gemm_tflops / tf_rand, 4),
+    }
+    if not args.skip_dense and N <= 16384:
+        hA, hB = dA.half(), dB.half()
+        for _ in range(3):
+            hC = torch.matmul(hA, hB)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            hC = torch.matmul(hA, hB)
+        e1.record()
+        torch.cuda.synchronize()
+        dense_ms = e0.elapsed_time(e1) / 5
+        out["dense_fp16_gemm"] = {
+            "library": "hipBLASLt via torch.matmul (fp16 in, fp16 out, conversion not timed)",
+            "ms": round(dense_ms, 4), "tflops": round(2.0 * N ** 3 / (dense_ms * 1e-3) / 1e12, 1),
+            "spamm_gemm_speedup": round(dense_ms / stage[3], 2),
+            "spamm_whole_multiply_speedup": round(dense_ms / ms_step, 2),
+        }
+        del hA, hB, hC
 
     # error against an exact fp64 dense product of the same fp16 operands, whole matrix, next to
     # the tau-derived bound (both formed on the device, outside the timed region)

@@ -72,6 +72,8 @@ def load_library():
     L.spamm_multiply_f16.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
     L.spamm_error_vs_dense_f64.argtypes = [vp, vp, i64, i64, ctypes.POINTER(ctypes.c_double)]
     L.spamm_dropped_bound.argtypes = [vp, f32, ctypes.POINTER(ctypes.c_double)]
+    L.spamm_mfma_ceiling.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                     ctypes.POINTER(ctypes.c_double)]
     L.spamm_load_csv_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
     L.spamm_load_mtx_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
     L.spamm_gate.argtypes = [vp, f32]
@@ -230,6 +232,13 @@ class SpammContext:
         _check(self._lib.spamm_error_vs_dense_f64(self._h, _devptr(C, "float32"), int(row0), int(row1), out),
                "spamm_error_vs_dense_f64")
         return out[0], out[1], out[2]
+
+    def mfma_ceiling(self, random_operands=True, iters=20000):
+        """(TFLOP/s, GHz) of a pure MFMA issue loop on every CU; a measurement aid."""
+        tf, ghz = ctypes.c_double(0), ctypes.c_double(0)
+        _check(self._lib.spamm_mfma_ceiling(self._h, int(bool(random_operands)), int(iters), ctypes.byref(tf),
+                                            ctypes.byref(ghz)), "spamm_mfma_ceiling")
+        return float(tf.value), float(ghz.value)
 
     def dropped_bound(self, tau):
         out = ctypes.c_double(0)

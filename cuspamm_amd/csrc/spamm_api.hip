@@ -415,6 +415,43 @@ int spamm_dropped_bound(spamm_ctx *c, float tau, double *out) {
     return SPAMM_OK;
 }
 
+int spamm_mfma_ceiling(spamm_ctx *c, int random_operands, int iters, double *tflops, double *clock_ghz) {
+    if (!c || !tflops || !clock_ghz || iters <= 0 || iters > (1 << 20)) return SPAMM_EINVAL;
+    int rc = set_device(c);
+    if (rc) return rc;
+    int n_wg = 0;
+    HIPCHK(c, hipDeviceGetAttribute(&n_wg, hipDeviceAttributeMultiprocessorCount, c->device));
+    if (n_wg <= 0 || n_wg > 4096) return SPAMM_EHIP;
+    // operands: 2048 vectors of 8 halves, zeros or uniform in [-1, 1) (a fixed LCG sequence)
+    std::vector<_Float16> h(2048 * 8);
+    uint32_t x = 12345u;
+    for (size_t i = 0; i < h.size(); i++) {
+        x = x * 1664525u + 1013904223u;
+        h[i] = random_operands ? (_Float16)(((float)(x >> 8) / 8388608.0f) - 1.0f) : (_Float16)0.0f;
+    }
+    const size_t in_bytes = h.size() * 2, out_bytes = (size_t)n_wg * 256 * 4, tr_bytes = (size_t)n_wg * 16;
+    if ((rc = ensure(c, c->scratch, in_bytes + out_bytes + tr_bytes))) return rc;
+    char *base = (char *)c->scratch.p;
+    HIPCHK(c, hipMemcpyAsync(base, h.data(), in_bytes, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    double best_ns = 0.0, best_clk = 0.0;
+    std::vector<unsigned long long> tr((size_t)n_wg * 2);
+    for (int rep = 0; rep < 3; rep++) {   // the clock settles over the first launches; keep the last
+        HIPCHK(c, launch_mfma_ceiling(base, (float *)(base + in_bytes), (unsigned long long *)(base + in_bytes + out_bytes),
+                                      n_wg, iters, c->stream));
+        if ((rc = copy_out(c, base + in_bytes + out_bytes, tr.data(), tr_bytes))) return rc;
+        double w = 0.0, k = 0.0;
+        for (int i = 0; i < n_wg; i++) { w += (double)tr[2 * i]; k += (double)tr[2 * i + 1]; }
+        best_ns = w / n_wg * 10.0;        // wall ticks are 10 ns
+        best_clk = k / n_wg;
+    }
+    if (best_ns <= 0.0) return SPAMM_EHIP;
+    const double flops = (double)iters * 16.0 * 32768.0 * 4.0 * n_wg;   // per MFMA 2*32*32*16, 4 waves per workgroup
+    *tflops = flops / best_ns * 1e-3;
+    *clock_ghz = best_clk / best_ns;
+    return SPAMM_OK;
+}
+
 // ---- input adapters (host side; getMatrixFromCSV / getMatrixFromMTX, tool.cu:282-366)
 static int load_text(const char *path, std::vector<char> &buf) {
     FILE *f = fopen(path, "rb");

@@ -30,7 +30,7 @@ inline int macro_dim(int tile) { return 256 / tile; }
 constexpr int SUPER_M = 4;
 constexpr int SUPER_N = 8;
 constexpr int NUM_XCD = 8;
-constexpr int SCHED_LEVELS = 4;   // work classes used to order macro tiles inside an XCD (0 = nothing kept)
+constexpr int SCHED_LEVELS = 2;   // work classes used to order macro tiles inside an XCD (0 = nothing kept)
 
 // Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin.
 inline int sched_rounds(int tile, int64_t nbM, int64_t nbN) {
@@ -78,6 +78,9 @@ hipError_t launch_error_vs_dense(const void *packedA, const void *packedB, int64
                                  hipStream_t s);
 hipError_t launch_dropped_bound(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
                                 float tau, double *out1, hipStream_t s);
+// matrix-pipeline ceiling probe: n_wg workgroups issue iters x 16 MFMAs per wave on the 32 KiB of operands at `in`
+hipError_t launch_mfma_ceiling(const void *in, float *out, unsigned long long *trace, int n_wg, int iters,
+                               hipStream_t s);
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,
                          uint16_t *out, hipStream_t s);
 hipError_t launch_transpose_normmap(const float *nB, int64_t nbK, int64_t nbN, float *nBt,

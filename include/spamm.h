@@ -173,6 +173,16 @@ SPAMM_API int spamm_error_vs_dense_f64(spamm_ctx *ctx, const float *dC, int64_t 
 /* tau-derived bound on that error: sqrt(sum_ij (sum_{k dropped} nA[i,k]*nB[k,j])^2). */
 SPAMM_API int spamm_dropped_bound(spamm_ctx *ctx, float tau, double *out);
 
+/* Measurement aid with no counterpart in the reference: the rate the matrix
+ * pipeline sustains when every CU issues nothing but independent fp16
+ * 32x32x16 MFMAs (iters x 16 per wave, one wave per SIMD), with all-zero
+ * operands (random_operands = 0) or uniform [-1,1) operands (1).  The
+ * sustained clock under MFMA load depends on the operand values, so the
+ * second figure is the ceiling a GEMM on real data can approach; it is
+ * reported next to the datasheet peak.  Synchronises. */
+SPAMM_API int spamm_mfma_ceiling(spamm_ctx *ctx, int random_operands, int iters, double *tflops,
+                                 double *clock_ghz);
+
 /* Input adapters (host): dense CSV, one matrix row per line (getMatrixFromCSV,
  * tool.cu:329-366), and "row col val" triples, 1-based, first line skipped
  * (getMatrixFromMTX, tool.cu:282-327).  host_out is rows x ld, zero-filled
