@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         const int64_t r0 = (int64_t)(mz / nMacN) * 256, c0 = (int64_t)(mz % nMacN) * 256 + lane * 4;
         if (c0 < N)
             for (int r = wave; r < 256 && r0 + r < M; r += 4)
-                *reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0) = zero;
+                __builtin_nontemporal_store(zero, reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0));
     };
     if (S == 0) {
         // nothing kept anywhere on this XCD's list (nc == 0): every workgroup zero-fills its own tile
@@ -354,7 +354,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     // ---- epilogue: C[row, col], row-major, ld N (cuSpAMM.cu:391).  MFMA
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
     // column l%32 of the block: every store instruction writes two full
-    // 128-byte row segments.  (Swapping the MFMA operands would give float4
+    // 128-byte row segments.  C is written once and not read again here:
+    // non-temporal stores leave the L2 to the operand panels.  (Swapping the MFMA operands would give float4
     // stores, but each then touches 32 rows with 32 bytes -- measured slower.)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
@@ -366,7 +367,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             if (col0 >= N) continue;
             float *out = C + (row0 + 4 * (lane >> 5)) * N + col0 + (lane & 31);
 #pragma unroll
-            for (int i = 0; i < 16; i++) out[(int64_t)(8 * (i / 4) + (i % 4)) * N] = acc[r][c][i];
+            for (int i = 0; i < 16; i++)
+                __builtin_nontemporal_store(acc[r][c][i], &out[(int64_t)(8 * (i / 4) + (i % 4)) * N]);
         }
     }
 
