@@ -145,6 +145,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         static_assert(G::LPW == 8, "the issue schedule below assumes 8 loads per wave per stage");
         const unsigned char *rowA[G::NG], *rowB[G::NG];
         uint32_t ldsA[G::NG];
+        int slot_of[G::NG];
 #pragma unroll
         for (int g = 0; g < G::NG; g++) {
             const int chunk0 = wave * G::CHW + g * G::GS;
@@ -155,12 +156,19 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             rowA[g] = pA + (int64_t)ti * nbK * G::TILE_BYTES + within0 * 1024;
             rowB[g] = pB + (int64_t)tj * nbK * G::TILE_BYTES + within0 * 1024;
             ldsA[g] = lds_base + slot * G::SLOT_BYTES + within0 * 1024;
+            slot_of[g] = slot;
         }
         const uint32_t voff = lane * 16;
 
         auto stage_k = [&](int t) -> uint32_t {
             const int tc = t < S ? t : S - 1;
             return ents[tc / G::NSPE].x;
+        };
+        // k and the needed-rows/columns bits of a stage's entry (one 8-byte scalar load)
+        typedef const __attribute__((address_space(4))) uint64_t *entry_kn_ptr;
+        auto stage_kn = [&](int t) -> uint64_t {
+            const int tc = t < S ? t : S - 1;
+            return *(entry_kn_ptr)(uintptr_t)(macro_list + (int64_t)macro * nbK + tc / G::NSPE);
         };
         // Load i (0..LPW-1) of a stage: i < CHW are the wave's A chunks, the
         // rest its B chunks.  A wave is in-order and alone on its SIMD, so a
@@ -187,15 +195,28 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 dma_load<j * 1024>(rowB[g] + sa.koff, voff, ldsA[g] + G::A_BYTES + sa.boff);
         };
 #define SPAMM_ISSUE(sa, i) issue_one(sa, std::integral_constant<int, i>{})
+        // Same load, but when no tile of the macro tile needs this operand slot at this k
+        // (need bit clear: the slot is never multiplied) the source is the first chunk of the
+        // operand array instead -- always valid and cache resident -- so that the number of
+        // loads in flight stays fixed while nothing is fetched for the slot.
+        auto issue_needed = [&](const StageAddr &sa, uint32_t need, auto idx) {
+            constexpr int i = decltype(idx)::value;
+            constexpr int op = i / G::CHW, ci = i % G::CHW;
+            constexpr int g = ci / G::GS, j = ci % G::GS;
+            if constexpr (op == 0) {
+                const unsigned char *src = ((need >> slot_of[g]) & 1u) ? rowA[g] + sa.koff : pA;
+                dma_load<j * 1024>(src, voff, ldsA[g] + sa.boff);
+            } else {
+                const unsigned char *src = ((need >> (8 + slot_of[g])) & 1u) ? rowB[g] + sa.koff : pB;
+                dma_load<j * 1024>(src, voff, ldsA[g] + G::A_BYTES + sa.boff);
+            }
+        };
+#define SPAMM_ISSUE_N(sa, nd, i) issue_needed(sa, nd, std::integral_constant<int, i>{})
         auto issue_all = [&](const StageAddr &sa) {
             SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); SPAMM_ISSUE(sa, 2); SPAMM_ISSUE(sa, 3);
             SPAMM_ISSUE(sa, 4); SPAMM_ISSUE(sa, 5); SPAMM_ISSUE(sa, 6); SPAMM_ISSUE(sa, 7);
         };
         auto issue_head = [&](const StageAddr &sa) { SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); };
-        auto issue_tail = [&](const StageAddr &sa) {
-            SPAMM_ISSUE(sa, 2); SPAMM_ISSUE(sa, 3); SPAMM_ISSUE(sa, 4);
-            SPAMM_ISSUE(sa, 5); SPAMM_ISSUE(sa, 6); SPAMM_ISSUE(sa, 7);
-        };
         // every wave: own loads of the next stage landed and own LDS reads
         // done; then the barrier makes both true for the whole workgroup
         auto sync_next = [&]() {
@@ -302,9 +323,11 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         SPAMM_TRACE(2);
         // ---- loop 2: entries kept by some tiles only; a wave multiplies
         // exactly the (tile row, tile column) pairs whose bit is set
+        uint32_t need_tail = 0xffffu;     // the stage whose head was issued by loop 1 / the prologue: all slots
         for (; t < S; t++) {
-            const uint32_t knext = stage_k(t + NBUF);
-            issue_tail(sa_tail);
+            const uint64_t kn = stage_kn(t + NBUF);
+            SPAMM_ISSUE_N(sa_tail, need_tail, 2); SPAMM_ISSUE_N(sa_tail, need_tail, 3); SPAMM_ISSUE_N(sa_tail, need_tail, 4);
+            SPAMM_ISSUE_N(sa_tail, need_tail, 5); SPAMM_ISSUE_N(sa_tail, need_tail, 6); SPAMM_ISSUE_N(sa_tail, need_tail, 7);
             const u32x4 cur = ents[t / G::NSPE];
             const uint64_t mask = ((uint64_t)cur.w << 32) | cur.z;
             uint32_t sb = 0;
@@ -337,14 +360,17 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 }
             }
             sync_next();
-            sa_tail = stage_addr(t + NBUF, knext);
-            issue_head(sa_tail);
+            sa_tail = stage_addr(t + NBUF, (uint32_t)kn);
+            // stages past the end repeat the last entry and are never read: nothing to fetch
+            need_tail = t + NBUF < S ? (uint32_t)(kn >> 32) : 0u;
+            SPAMM_ISSUE_N(sa_tail, need_tail, 0); SPAMM_ISSUE_N(sa_tail, need_tail, 1);
         }
 #undef SPAMM_MFMA
 #undef SPAMM_FENCE
 #undef SPAMM_LDA
 #undef SPAMM_LDB
 #undef SPAMM_ISSUE
+#undef SPAMM_ISSUE_N
         SPAMM_TRACE(3);
         // the ring still holds clamped loads: let them land before the
         // workgroup gives its LDS back
