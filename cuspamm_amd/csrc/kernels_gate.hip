@@ -44,22 +44,36 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         const float *rb = g.nBt + (int64_t)j * nbK;
         const int64_t tid = (int64_t)i * nbN + j;
         int base = 0;
-        for (int w = 0; w < words; w++) {
-            const int k = w * 64 + lane;
-            bool keep = false;
-            if (inside && k < nbK) {
-                const float p = ra[k] * rb[k];
-                keep = p >= tau;
+        // four 64-k words per step: their norm loads are in flight together (each is a cache round trip)
+        for (int w0 = 0; w0 < words; w0 += 4) {
+            float pa[4], pb[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int k = (w0 + u) * 64 + lane;
+                const bool live = inside && k < nbK;
+                pa[u] = live ? ra[k] : 0.0f;
+                pb[u] = live ? rb[k] : 0.0f;
             }
-            const uint64_t m = __ballot(keep);
-            if (keep) {
-                const int pos = base + __builtin_popcountll(m & ((1ull << lane) - 1ull));
-                g.klist[tid * nbK + pos] = (uint16_t)k;
-            }
-            base += __builtin_popcountll(m);
-            if (lane == 0) {
-                lmask[(size_t)t * words + w] = m;
-                if (inside) g.mask[tid * words + w] = m;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int w = w0 + u;
+                if (w >= words) break;
+                const int k = w * 64 + lane;
+                bool keep = false;
+                if (inside && k < nbK) {
+                    const float p = pa[u] * pb[u];
+                    keep = p >= tau;
+                }
+                const uint64_t m = __ballot(keep);
+                if (keep) {
+                    const int pos = base + __builtin_popcountll(m & ((1ull << lane) - 1ull));
+                    g.klist[tid * nbK + pos] = (uint16_t)k;
+                }
+                base += __builtin_popcountll(m);
+                if (lane == 0) {
+                    lmask[(size_t)t * words + w] = m;
+                    if (inside) g.mask[tid * words + w] = m;
+                }
             }
         }
         if (inside && lane == 0) g.counts[tid] = base;
@@ -259,14 +273,23 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         const int x = wave;
         const int32_t *rx = raw + x * P;
         int mycnt = 0;                       // lane lv < SCHED_LEVELS keeps the count of level lv
-        for (int p0 = 0; p0 < P; p0 += 64) {
-            const int p = p0 + lane;
-            const int v = p < P ? rx[p] : -1;
-            const int level = v >= 0 ? (v >> 24) : -1;
+        // (loads of UN chunks are issued together: the wave is alone here and each one is an L2 round trip)
+        constexpr int UN = 8;
+        for (int p0 = 0; p0 < P; p0 += 64 * UN) {
+            int vv[UN];
 #pragma unroll
-            for (int lv = 0; lv < SCHED_LEVELS; lv++) {
-                const int c = __builtin_popcountll(__ballot(level == lv));
-                if (lane == lv) mycnt += c;
+            for (int u = 0; u < UN; u++) {
+                const int p = p0 + u * 64 + lane;
+                vv[u] = p < P ? rx[p] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int level = vv[u] >= 0 ? (vv[u] >> 24) : -1;
+#pragma unroll
+                for (int lv = 0; lv < SCHED_LEVELS; lv++) {
+                    const int c = __builtin_popcountll(__ballot(level == lv));
+                    if (lane == lv) mycnt += c;
+                }
             }
         }
         // exclusive prefix over levels in descending order: base(lv) = sum of counts of levels > lv
@@ -282,19 +305,27 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
             g.sched[x] = ncomp;
             g.sched[NUM_XCD + x] = nall;
         }
-        for (int p0 = 0; p0 < P; p0 += 64) {
-            const int p = p0 + lane;
-            const int v = p < P ? rx[p] : -1;
-            const int level = v >= 0 ? (v >> 24) : -1;
-            int pos = -1;
+        for (int p0 = 0; p0 < P; p0 += 64 * UN) {
+            int vv[UN];
 #pragma unroll
-            for (int lv = 0; lv < SCHED_LEVELS; lv++) {
-                const uint64_t bal = __ballot(level == lv);
-                const int b0 = __shfl(base, lv, 64);
-                if (level == lv) pos = b0 + __builtin_popcountll(bal & ((1ull << lane) - 1ull));
-                if (lane == lv) base += __builtin_popcountll(bal);
+            for (int u = 0; u < UN; u++) {
+                const int p = p0 + u * 64 + lane;
+                vv[u] = p < P ? rx[p] : -1;
             }
-            if (pos >= 0) g.order[x * P + pos] = v & 0xffffff;
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int v = vv[u];
+                const int level = v >= 0 ? (v >> 24) : -1;
+                int pos = -1;
+#pragma unroll
+                for (int lv = 0; lv < SCHED_LEVELS; lv++) {
+                    const uint64_t bal = __ballot(level == lv);
+                    const int b0 = __shfl(base, lv, 64);
+                    if (level == lv) pos = b0 + __builtin_popcountll(bal & ((1ull << lane) - 1ull));
+                    if (lane == lv) base += __builtin_popcountll(bal);
+                }
+                if (pos >= 0) g.order[x * P + pos] = v & 0xffffff;
+            }
         }
     }
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;
