@@ -199,8 +199,8 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 //      kept) the computing macro tiles simply run super tile by super tile:
 //      measured on banded inputs, finer heaviest-first classes did not
 //      shorten the tail but pulled neighbours apart (10 % more L2 misses).
-//   3. Macro tiles with nothing kept come last in each XCD's sequence; the
-//      computing workgroups zero-fill them after their own epilogue.
+//   3. Macro tiles with nothing kept come last in each XCD's sequence: their
+//      workgroups only write zeros and start when CUs fall idle at the end.
 // Output: order[x * P + q] = macro tile id of XCD x's q-th workgroup,
 // sched[x] = number of computing items, sched[8 + x] = number of all items.
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.

@@ -96,13 +96,13 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const int wr = wave >> 1, wc = wave & 1;
     // Workgroup b runs on XCD b % NUM_XCD and is that XCD's q-th workgroup,
     // q = b / NUM_XCD; `order` holds each XCD's sequence: computing macro tiles
-    // (heaviest level first), then the ones with nothing kept.  A computing
-    // workgroup afterwards zero-fills its share of the latter (q + nc,
-    // q + 2 nc, ...), so those stores drain while other workgroups compute.
+    // first, then the ones with nothing kept.  The latter's workgroups only
+    // write zeros; they are dispatched when CUs start to fall idle at the end
+    // of the XCD's queue, so the zero-fill fills the tail of the kernel
+    // instead of competing with the k loops for memory bandwidth.
     const int xcd = blockIdx.x % NUM_XCD, q = blockIdx.x / NUM_XCD;
-    const int nc = __builtin_amdgcn_readfirstlane(sched[xcd]);
     const int ntot = __builtin_amdgcn_readfirstlane(sched[NUM_XCD + xcd]);
-    if (q >= ntot || (nc > 0 && q >= nc)) return;
+    if (q >= ntot) return;
     SPAMM_TRACE(0);
     const int32_t *seq = order + (int64_t)xcd * P;
     const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
@@ -122,8 +122,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 __builtin_nontemporal_store(zero, reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0));
     };
     if (S == 0) {
-        // nothing kept anywhere on this XCD's list (nc == 0): every workgroup zero-fills its own tile
-        zero_fill(macro);
+        zero_fill(macro);     // q >= nc: nothing kept in this macro tile
         return;
     }
 
@@ -399,7 +398,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     }
 
     // ---- zero-fill this workgroup's share of the macro tiles with nothing kept
-    for (int e = nc + q; e < ntot; e += nc) zero_fill(__builtin_amdgcn_readfirstlane(seq[e]));
 #ifdef SPAMM_EXP_TRACE
     SPAMM_TRACE(4);
     if (threadIdx.x == 0) {
