@@ -1,7 +1,10 @@
-"""BASELINE-sized runs (N = 16384, tile 64): bit-exact mask over the whole
-problem, C against the checker and against an exact fp64 product on sampled
-tile rows, plus size-independent properties (all-ones closed form, exact
-power-of-two scaling, kept count == popcount of the mask)."""
+"""BASELINE-sized runs (N = 8192 / 16384, tile 64; N = 65536, tile 128): bit-exact
+mask over the whole problem, C against the checker and against an exact fp64
+product on sampled tile rows, plus size-independent properties (all-ones closed
+form, exact power-of-two scaling, kept count == popcount of the mask).  At
+N = 65536 the host never holds the matrices: the mask is checked against the
+checker's gate on the read-back norm maps, the norm maps by closed forms and the
+Frobenius invariant, C by the device's fp64 dense comparison."""
 import numpy as np
 import pytest
 
@@ -10,11 +13,11 @@ pytestmark = pytest.mark.gpu
 N = 16384
 TILE = 64
 C_REL_TOL = 1e-3
-SAMPLE_ROWS = [0, 97, 255]          # tile rows checked element-wise on the host
 
 
-def _full_case(orc, ctx, kind, lam, ratio=None, tau=None):
+def _full_case(orc, ctx, kind, lam, ratio=None, tau=None, N=N):
     import torch
+    sample_rows = [0, (N // TILE) // 3 + 12, N // TILE - 1]
     tab = orc.decay_table(kind, N, lam)
     dA = torch.empty((N, N), dtype=torch.float32, device="cuda")
     dB = torch.empty((N, N), dtype=torch.float32, device="cuda")
@@ -41,7 +44,7 @@ def _full_case(orc, ctx, kind, lam, ratio=None, tau=None):
     Af, Bf = orc.f16_bits_to_f32(hA), orc.f16_bits_to_f32(hB)
     del hA, hB
     Cref = np.zeros((N, N), dtype=np.float32)
-    for ti in SAMPLE_ROWS:
+    for ti in sample_rows:
         orc.gemm_gated(Af, Bf, TILE, counts, klist, ti0=ti, ti1=ti + 1, out=Cref)
         rows = slice(ti * TILE, (ti + 1) * TILE)
         Cg = C[rows].cpu().numpy()
@@ -60,6 +63,12 @@ def _full_case(orc, ctx, kind, lam, ratio=None, tau=None):
 def test_headline_exponential_decay_ten_percent(orc, ctx):
     kept = _full_case(orc, ctx, "exp", 0.003, ratio=0.10)
     assert abs(kept / 256 ** 3 - 0.10) < 0.01
+
+
+def test_config2_n8192_ten_percent(orc, ctx):
+    # exp(-0.1 d) cannot keep 10 % after fp16 rounding (at most 0.29 %); lam = 0.01 can
+    kept = _full_case(orc, ctx, "exp", 0.01, ratio=0.10, N=8192)
+    assert abs(kept / 128 ** 3 - 0.10) < 0.01
 
 
 def test_config3_algebraic_decay_twenty_percent(orc, ctx):
@@ -111,3 +120,56 @@ def test_power_of_two_scaling_is_exact(orc, ctx):
     assert torch.equal(C2, 2 * C1)
     frac = np.unpackbits(m1.view(np.uint8)).sum() / 256 ** 3
     assert 0.05 < frac < 0.2
+
+
+N5, TILE5 = 65536, 128
+
+
+def test_config5_n65536_tile128_two_percent(orc, ctx):
+    import torch
+    nb = N5 // TILE5
+    tab = orc.decay_table("exp", N5, 0.003)
+    dA = torch.empty((N5, N5), dtype=torch.float32, device="cuda")
+    dB = torch.empty((N5, N5), dtype=torch.float32, device="cuda")
+    ctx.fill_decay(dA, tab, 1)
+    ctx.fill_decay(dB, tab, 2)
+    ctx.normmap_f32(1, dB, TILE5)
+    ctx.normmap_f32(0, dA, TILE5)
+    tau, ach = ctx.tau_for_ratio(0.02)
+    assert abs(ach - 0.02) < 0.002
+    C = ctx.multiply(dA, dB, TILE5, tau)
+    nA, nB = ctx.get_normmap(0), ctx.get_normmap(1)
+    # Frobenius invariant of the norm maps against the fp16-rounded inputs (row blocks, fp64)
+    for X, nm in ((dA, nA), (dB, nB)):
+        tot = 0.0
+        for r0 in range(0, N5, 4096):
+            tot += float((X[r0:r0 + 4096].half().double() ** 2).sum())
+        assert abs(float((nm.astype(np.float64) ** 2).sum()) - tot) <= 1e-6 * tot
+    del dA, dB
+    kept, counts, klist, mask = orc.gate(nA, nB, tau)
+    gmask = ctx.get_mask()
+    assert np.array_equal(gmask, mask)                                    # bit-exact kept mask, 1.3e8 products
+    assert np.array_equal(ctx.get_counts(), counts)
+    st = ctx.get_stats()
+    assert st.kept_products == kept and st.total_products == nb ** 3
+    assert abs(kept / nb ** 3 - 0.02) < 0.002
+    # C against the exact fp64 product of the resident fp16 operands, on two row slabs
+    bound = ctx.dropped_bound(tau)
+    for r0 in (0, 30080):
+        err, dense, cn = ctx.error_vs_dense(C, r0, r0 + 128)
+        assert dense > 0 and err <= bound * (1 + 1e-4) + 1e-5 * dense
+        assert err <= 1e-3 * dense
+    zero_rows = C.view(nb, TILE5, nb, TILE5).abs().amax(dim=(1, 3)).cpu().numpy()
+    assert np.all(zero_rows[counts == 0] == 0)
+    assert np.all(zero_rows[counts > 0] > 0)
+
+
+def test_all_ones_closed_form_n65536(ctx):
+    import torch
+    ones = torch.ones((N5, N5), dtype=torch.float32, device="cuda")
+    ctx.normmap_f32(0, ones, TILE5)
+    assert np.all(ctx.get_normmap(0) == float(TILE5))                     # sqrt(128 * 128) exactly
+    C = ctx.multiply(ones, ones, TILE5, 0.0)
+    assert ctx.get_stats().kept_products == (N5 // TILE5) ** 3
+    for r0 in range(0, N5, 8192):
+        assert bool(torch.all(C[r0:r0 + 8192] == N5))
