@@ -126,7 +126,7 @@ SPAMM_API int spamm_gemm_gated(spamm_ctx *ctx, float *dC);
  *     >= tau are kept (ties may push the achieved ratio above the target); if
  *     fewer positive products exist, the smallest positive one.
  *   spamm_tune_bisect: the reference's bisection, same arithmetic
- *     (tool.cu:445-486): round 0 measures the ratio at tau = 0 and moves to the
+ *     (tool.cu:445-486): iteration 0 measures the ratio at tau = 0 and moves to the
  *     mean product, later rounds bisect, stop at |ratio - expected| < tol or
  *     after max_rounds (reference: 0.75, 0.01, 20).  Counting runs on the device.
  *   spamm_count_kept: products with (double)product >= threshold, and the

@@ -398,7 +398,7 @@ ORC_API float orc_tau_for_ratio(const float *nA, const float *nB, int64_t nbM, i
     return tau;
 }
 
-/* The reference's bisection (tool.cu:438-490): round 0 measures the ratio at
+/* The reference's bisection (tool.cu:438-490): iteration 0 measures the ratio at
  * tau = 0 and sets tau to the mean product; later rounds bisect between
  * down/up, doubling `up` while the ratio is still too high; stops when
  * |ratio - expected| < tol or after max_rounds.  Products and comparisons are
