@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     __syncthreads();
     // inclusive scans over words (Hillis-Steele in LDS; words is small)
     for (int off = 1; off <= words; off <<= 1) {
-        int addf[4], addp[4];
+        int addf[5], addp[5];        // words <= 1024: at most 5 per thread
         int n = 0;
         for (int w = threadIdx.x; w <= words; w += 256) {
             addf[n] = w >= off ? wfull[w - off] : 0;
@@ -335,6 +335,12 @@ size_t gate_lds_bytes(int tile, int64_t nbK) {
     const int MT = macro_dim(tile);
     const size_t words = (size_t)((nbK + 63) / 64);
     return (size_t)MT * MT * words * 8 + 2 * (words + 1) * 4 + 8;
+}
+
+// k_gate may use all of a CU's LDS for the macro tile's bitmaps (its workgroups are short)
+hipError_t gate_init() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)gate_lds_limit());
 }
 
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,

@@ -161,7 +161,7 @@ int spamm_create(spamm_ctx **out, int device) {
     c->stream = c->own_stream;
     for (int i = 0; i < 5 && rc == SPAMM_OK; i++)
         if (hipEventCreate(&c->ev[i]) != hipSuccess) rc = SPAMM_EHIP;
-    if (rc == SPAMM_OK && gemm_init() != hipSuccess) rc = SPAMM_EHIP;
+    if (rc == SPAMM_OK && (gemm_init() != hipSuccess || gate_init() != hipSuccess)) rc = SPAMM_EHIP;
     if (rc != SPAMM_OK) {
         (void)hipGetLastError();
         spamm_destroy(c);          // releases whatever was created
@@ -280,7 +280,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
     int rc = set_device(c);
     if (rc) return rc;
     const Shape s = shape_of(c);
-    if (gate_lds_bytes(c->tile, s.nbK) > 64 * 1024) return SPAMM_EINVAL;
+    if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // K / tile beyond ~20 000 (tile 32)
     const size_t nt = (size_t)s.nbM * s.nbN;
     if ((rc = ensure(c, c->counts, nt * 4))) return rc;
     if ((rc = ensure(c, c->klist, nt * s.nbK * 2))) return rc;

@@ -89,6 +89,8 @@ hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *
                              uint64_t seed, int random, hipStream_t s);
 
 size_t gate_lds_bytes(int tile, int64_t nbK);
+inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k_gate (a few static bytes aside)
+hipError_t gate_init();   // one-time kernel attribute set-up
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
                        float tau, hipStream_t s);
 
