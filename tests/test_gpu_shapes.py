@@ -46,7 +46,8 @@ def test_random_shapes(orc, ctx):
                                         (128, 32768, 128, 128), (2560, 256, 2304, 64), (32, 32, 32, 32),
                                         (288, 32, 2080, 32),
                                         (64, 576, 102400, 64),     # the reference's im2col shape (para.h:20-21)
-                                        (32, 288000, 32, 32)])     # 9000 k tiles: bitmaps beyond 64 KiB of LDS
+                                        (32, 288000, 32, 32),      # 9000 k tiles: bitmaps beyond 64 KiB of LDS
+                                        (64, 65535 * 64, 64, 64)])  # the most k tiles the ABI takes
 def test_extreme_aspect_ratios(orc, ctx, M, K, N, tile):
     tab = orc.decay_table("exp", max(M, K, N), 0.002)
     A = orc.fill_decay(M, K, tab, 1)
