@@ -18,6 +18,7 @@ namespace spamm {
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4n __attribute__((ext_vector_type(4)));
 
 // Convert two floats to fp16 (round-to-nearest-even), add their squares to s
 // in order (a then b) and return the packed pair.
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             if (Jt < nbc) {
                 const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
                 const int64_t tile = as_b ? Jt * nbr + I : I * nbc + Jt;
-                pk[tile * VPT + iv] = d;
+                __builtin_nontemporal_store(*reinterpret_cast<const u32x4n *>(&d), reinterpret_cast<u32x4n *>(pk + tile * VPT + iv));
             }
         }
         for (int tt = wave; tt < TPS; tt += 4) {
