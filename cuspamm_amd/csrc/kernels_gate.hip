@@ -47,6 +47,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         // four 64-k words per step: their norm loads are in flight together (each is a cache round trip)
         for (int w0 = 0; w0 < words; w0 += 4) {
             float pa[4], pb[4];
+            uint64_t mword = 0;
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int k = (w0 + u) * 64 + lane;
@@ -70,10 +71,12 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
                     g.klist[tid * nbK + pos] = (uint16_t)k;
                 }
                 base += __builtin_popcountll(m);
-                if (lane == 0) {
-                    lmask[(size_t)t * words + w] = m;
-                    if (inside) g.mask[tid * words + w] = m;
-                }
+                if (lane == u) mword = m;              // lane u keeps word w0 + u
+            }
+            // one store of up to four words per step instead of one per word
+            if (lane < 4 && w0 + lane < words) {
+                lmask[(size_t)t * words + w0 + lane] = mword;
+                if (inside) g.mask[tid * words + w0 + lane] = mword;
             }
         }
         if (inside && lane == 0) g.counts[tid] = base;
