@@ -8,7 +8,7 @@
 // of C; each wave owns 128 x 128 (4 x 4 MFMA 32x32x16 accumulators = 256 fp32
 // registers per lane).  The workgroup walks the macro tile's union list of k;
 // per entry it stages the needed A tiles (256 rows) and B tiles (256 columns)
-// of that k in LDS with direct global->LDS loads, double buffered, and every
+// of that k in LDS with direct global->LDS loads (a ring of NBUF stages), and every
 // wave multiplies only the (tile row, tile column) pairs whose bit is set in
 // the entry's mask, so the kept set is exactly the gate's.
 //
