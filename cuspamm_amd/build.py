@@ -11,6 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libspamm_gfx950.so")
+MAIN_PATH = os.path.join(HERE, "spamm_main")     # the reference's main() on top of the C ABI (csrc/spamm_main.cpp)
 
 SOURCES = ["kernels_normmap.hip", "kernels_gate.hip", "kernels_gemm.hip", "kernels_tau.hip", "kernels_tools.hip",
            "spamm_api.hip"]
@@ -83,6 +84,8 @@ def build_library(verbose=False):
     with ThreadPoolExecutor(max_workers=4) as ex:
         logs = list(ex.map(compile_one, zip(SOURCES, objs)))
     logs.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs))
+    logs.append(_run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wall", os.path.join(CSRC, "spamm_main.cpp"), "-o", MAIN_PATH,
+                      "-L" + HERE, "-lspamm_gfx950", "-Wl,-rpath,$ORIGIN"]))
     if verbose:
         for text in logs:
             if text.strip():

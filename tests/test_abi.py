@@ -69,6 +69,17 @@ def test_create_without_gpu_reports_no_device():
     assert ei.value.code == -5
 
 
+def test_command_line_driver_is_built_and_checks_its_arguments():
+    # argument errors are reported before any device call, so this runs without a GPU
+    import subprocess
+    main = os.path.join(ROOT, "cuspamm_amd", "spamm_main")
+    assert os.path.exists(main), "build it with `python -m cuspamm_amd.build`"
+    for args, msg in ((["--tile", "48"], "tile must be"), (["--nonsense"], "unknown option"),
+                      (["--testtime", "3", "--warmup", "5"], "bad sizes")):
+        proc = subprocess.run([main] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+        assert proc.returncode == 2 and msg in proc.stdout, proc.stdout
+
+
 def test_product_package_never_imports_the_oracle():
     # the checker is test infrastructure: nothing under cuspamm_amd/ may reference it
     pkg = os.path.join(ROOT, "cuspamm_amd")
