@@ -28,13 +28,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#ifdef SPAMM_EXP_TRACE
-__device__ unsigned long long g_trace[16384 * 8];
-#define SPAMM_TRACE(slot) do { if (threadIdx.x == 0) { g_trace[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64(); if ((slot) == 1) g_trace[(size_t)blockIdx.x * 8 + 7] = clock64(); if ((slot) == 2) g_trace[(size_t)blockIdx.x * 8 + 7] = clock64() - g_trace[(size_t)blockIdx.x * 8 + 7]; } } while (0)
-#else
-#define SPAMM_TRACE(slot) do { } while (0)
-#endif
-
 template <int B>
 struct GemmCfg {
     static constexpr int SUB = 128 / B;              // tiles per wave per dimension
@@ -103,7 +96,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const int xcd = blockIdx.x % NUM_XCD, q = blockIdx.x / NUM_XCD;
     const int ntot = __builtin_amdgcn_readfirstlane(sched[NUM_XCD + xcd]);
     if (q >= ntot) return;
-    SPAMM_TRACE(0);
     const int32_t *seq = order + (int64_t)xcd * P;
     const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
     const int mi = macro / nMacN, mj = macro % nMacN;
@@ -249,8 +241,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         issue_head(sa_tail);
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2) + 2, 0));
         __syncthreads();
-
-        SPAMM_TRACE(1);
         int t = 0;
         // ---- loop 1: entries kept by all tiles of the macro tile; no
         // branches.  Operand vectors are double buffered in registers (a0/b0:
@@ -263,9 +253,9 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 #define SPAMM_FENCE() __builtin_amdgcn_sched_barrier(0)
 #define SPAMM_LDA(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufA + frag_off(wr, blk, kk))
 #define SPAMM_LDB(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufB + frag_off(wc, blk, kk))
+        half8 a0[4], b0[4], a1[4], b1[4];
+        load_frags(a0, b0, 0, 0);
         if (Sfull > 0) {
-            half8 a0[4], b0[4], a1[4], b1[4];
-            load_frags(a0, b0, 0, 0);
             uint32_t knext = stage_k(NBUF);
             for (; t < Sfull; t++) {
                 // address of the stage issued after this iteration's sync, computed early so that
@@ -319,9 +309,26 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 }
             }
         }
-        SPAMM_TRACE(2);
         // ---- loop 2: entries kept by some tiles only; a wave multiplies
-        // exactly the (tile row, tile column) pairs whose bit is set
+        // exactly the (tile row, tile column) pairs whose bit is set.  Same
+        // register double buffering as loop 1: on entry a0/b0 hold k step 0
+        // of stage t; k step 1 is read while step 0 multiplies, and the next
+        // stage's step 0 (readable after the sync) while step 1 multiplies.
+        auto mul_kept = [&](const half8 (&af)[4], const half8 (&bf)[4], uint32_t sb) {
+#pragma unroll
+            for (int a = 0; a < G::SUB; a++)
+#pragma unroll
+                for (int b = 0; b < G::SUB; b++) {
+                    if ((sb >> (a * G::SUB + b)) & 1u) {
+#pragma unroll
+                        for (int r = 0; r < G::RB; r++)
+#pragma unroll
+                            for (int c = 0; c < G::RB; c++)
+                                acc[a * G::RB + r][b * G::RB + c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                                    af[a * G::RB + r], bf[b * G::RB + c], acc[a * G::RB + r][b * G::RB + c], 0, 0, 0);
+                    }
+                }
+        };
         uint32_t need_tail = 0xffffu;     // the stage whose head was issued by loop 1 / the prologue: all slots
         for (; t < S; t++) {
             const uint64_t kn = stage_kn(t + NBUF);
@@ -337,32 +344,15 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                     const int bit = (wr * G::SUB + a) * G::MT + wc * G::SUB + b;
                     sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
                 }
-            if (sb != 0) {
-#pragma unroll
-                for (int kk = 0; kk < 2; kk++) {
-                    half8 af[4], bf[4];
-                    load_frags(af, bf, t, kk);
-#pragma unroll
-                    for (int a = 0; a < G::SUB; a++)
-#pragma unroll
-                        for (int b = 0; b < G::SUB; b++) {
-                            if ((sb >> (a * G::SUB + b)) & 1u) {
-#pragma unroll
-                                for (int r = 0; r < G::RB; r++)
-#pragma unroll
-                                    for (int c = 0; c < G::RB; c++)
-                                        acc[a * G::RB + r][b * G::RB + c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                                            af[a * G::RB + r], bf[b * G::RB + c], acc[a * G::RB + r][b * G::RB + c], 0,
-                                            0, 0);
-                            }
-                        }
-                }
-            }
+            load_frags(a1, b1, t, 1);
+            mul_kept(a0, b0, sb);
             sync_next();
             sa_tail = stage_addr(t + NBUF, (uint32_t)kn);
             // stages past the end repeat the last entry and are never read: nothing to fetch
             need_tail = t + NBUF < S ? (uint32_t)(kn >> 32) : 0u;
             SPAMM_ISSUE_N(sa_tail, need_tail, 0); SPAMM_ISSUE_N(sa_tail, need_tail, 1);
+            load_frags(a0, b0, t + 1, 0);
+            mul_kept(a1, b1, sb);
         }
 #undef SPAMM_MFMA
 #undef SPAMM_FENCE
@@ -370,7 +360,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 #undef SPAMM_LDB
 #undef SPAMM_ISSUE
 #undef SPAMM_ISSUE_N
-        SPAMM_TRACE(3);
         // the ring still holds clamped loads: let them land before the
         // workgroup gives its LDS back
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
@@ -380,8 +369,9 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
     // column l%32 of the block: every store instruction writes two full
     // 128-byte row segments.  C is written once and not read again here:
-    // non-temporal stores leave the L2 to the operand panels.  (Swapping the MFMA operands would give float4
-    // stores, but each then touches 32 rows with 32 bytes -- measured slower.)
+    // non-temporal stores leave the L2 to the operand panels.  (Swapping the
+    // MFMA operands would give float4 stores, but each then touches 32 rows
+    // with 32 bytes -- measured slower.)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const int64_t row0 = (int64_t)mi * 256 + wr * 128 + r * 32;
@@ -396,18 +386,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                 __builtin_nontemporal_store(acc[r][c][i], &out[(int64_t)(8 * (i / 4) + (i % 4)) * N]);
         }
     }
-
-    // ---- zero-fill this workgroup's share of the macro tiles with nothing kept
-#ifdef SPAMM_EXP_TRACE
-    SPAMM_TRACE(4);
-    if (threadIdx.x == 0) {
-        unsigned hwid, xccid;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xccid));
-        g_trace[(size_t)blockIdx.x * 8 + 5] = ((unsigned long long)xccid << 32) | hwid;
-        g_trace[(size_t)blockIdx.x * 8 + 6] = (unsigned long long)S | ((unsigned long long)Sfull << 32);
-    }
-#endif
 }
 
 static int g_nbuf = 4;
@@ -469,11 +447,5 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     }
     return hipGetLastError();
 }
-
-#ifdef SPAMM_EXP_TRACE
-extern "C" __attribute__((visibility("default"))) int spamm_debug_trace(void *host, size_t bytes) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), bytes);
-}
-#endif
 
 }  // namespace spamm
