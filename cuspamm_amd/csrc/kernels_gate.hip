@@ -5,121 +5,221 @@
 // (fp32 multiply, fp32 compare, :305-306), serial O(n^2) compaction
 // (:315-325) and a shared-memory tree count (:328-334).  Here one workgroup
 // owns one macro tile (256 x 256 elements of C = MT x MT output tiles):
-//   phase 1  each wave takes output tiles of the macro tile in turn; 64 k per
-//            ballot, popcount/mbcnt gives every kept k its slot in the
-//            ascending list; per-tile bitmap, list and count go to memory and
-//            the bitmap words also to LDS;
-//   phase 2  union of the MT*MT bitmaps per 64-k word, popcount per word, an
-//            LDS prefix sum over the words, then every kept k of the union is
-//            written at its prefix position together with the bit set of
-//            tiles that keep it.  The union list is what the gated GEMM walks;
-//            its length and the kept-product total are the work counts used to
-//            order macro tiles for load balance.
+//   phase 1  a wave takes a block of up to 4 x 4 output tiles and 64 k at a
+//            time: it loads the 4 + 4 norms once per lane, forms the 16
+//            products in registers and ballots each comparison into the
+//            tile's 64-bit bitmap word, kept in LDS;
+//   phase 2  per-tile counts and the bitmaps go to memory; then every 64-k
+//            word of the MT*MT bitmaps is transposed across a wave (lane =
+//            k), which gives each k the bit set of tiles that keep it, the
+//            union and the kept-by-all word; an LDS prefix sum over the words
+//            places every kept k of the union in the macro tile's list.  The
+//            union list is what the gated GEMM walks; its length and the
+//            kept-product total are the work counts used to order macro tiles
+//            for load balance.
+// The reference's compacted per-tile list (offset[], :315-325) is the bitmap's
+// set bits in ascending order; nothing downstream reads it, so it is produced
+// from the bitmap only when asked for (k_klist).
 #include "spamm_internal.h"
 
 namespace spamm {
 
-__global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int MT,
-                                              int nMacN, float tau) {
+// 64 x 64 bit-matrix transpose across a wave: lane t holds row t; on return
+// lane b holds column b (bit t of the result = bit b of lane t's input).
+// Six butterfly steps, each swapping the off-diagonal j x j blocks of lane
+// pairs (l, l ^ j).
+__device__ __forceinline__ uint64_t transpose64(uint64_t x, int lane) {
+    constexpr uint64_t MASKS[6] = {0x00000000FFFFFFFFull, 0x0000FFFF0000FFFFull, 0x00FF00FF00FF00FFull,
+                                   0x0F0F0F0F0F0F0F0Full, 0x3333333333333333ull, 0x5555555555555555ull};
+#pragma unroll
+    for (int s = 0; s < 6; s++) {
+        const int j = 32 >> s;
+        const uint64_t y = (uint64_t)__shfl_xor((long long)x, j, 64);
+        const bool upper = (lane & j) == 0;              // this lane is the row without bit j
+        const uint64_t ru = upper ? x : y, rl = upper ? y : x;
+        const uint64_t t = ((ru >> j) ^ rl) & MASKS[s];
+        x ^= upper ? (t << j) : t;
+    }
+    return x;
+}
+
+// v[lane idx] = s for a wave-uniform s; idx must fold to a constant (unrolled loops)
+__device__ __forceinline__ void set_lane(int &v, uint32_t s, int idx) {
+    asm("v_writelane_b32 %0, %1, %2" : "+v"(v) : "s"(s), "n"(idx));
+}
+
+template <int MT>
+struct GateCfg {
+    static constexpr int NT = MT * MT;             // output tiles per macro tile
+    static constexpr int NTP = NT < 8 ? 8 : NT;    // bitmap rows per 64-k word in LDS (a transposed word needs 64 * NTP bits)
+    static constexpr int BT = MT < 4 ? MT : 4;     // a wave's block of tiles per dimension
+    static constexpr int QD = MT / BT;
+    static constexpr int NQ = QD * QD;
+    static constexpr uint64_t FULL = NT == 64 ? ~0ull : ((1ull << NT) - 1ull);
+};
+
+template <int MT>
+__global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int nMacN, float tau) {
+    using G = GateCfg<MT>;
+    constexpr int NT = G::NT, NTP = G::NTP, BT = G::BT;
     extern __shared__ uint64_t smem[];
     const int words = (nbK + 63) >> 6;
-    const int NT = MT * MT;
-    uint64_t *lmask = smem;                                   // [NT][words]
-    int *wsum = reinterpret_cast<int *>(smem + (size_t)NT * words);   // 2 x [words + 1] prefixes
-    __shared__ int s_work;
+    uint64_t *lmask = smem;                                  // [words][NTP]: tile bitmaps, later transposed in place
+    uint64_t *luf = smem + (size_t)words * NTP;              // [words][2]: union word, kept-by-all word
+    int *wfull = reinterpret_cast<int *>(luf + 2 * (size_t)words);   // [words + 1] prefix of full entries
+    int *wpart = wfull + (words + 1);                        // [words + 1] prefix of partial entries
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int macro = blockIdx.x;
     const int mi = macro / nMacN, mj = macro % nMacN;
-    if (threadIdx.x == 0) s_work = 0;
-    __syncthreads();
 
-    // ---- phase 1: per output tile bitmap + ascending list + count
-    int my_work = 0;
-    for (int t = wave; t < NT; t += 4) {
-        const int i = mi * MT + t / MT, j = mj * MT + t % MT;
-        const bool inside = i < nbM && j < nbN;
-        const float *ra = g.nA + (int64_t)i * nbK;
-        const float *rb = g.nBt + (int64_t)j * nbK;
-        const int64_t tid = (int64_t)i * nbN + j;
-        int base = 0;
-        // four 64-k words per step: their norm loads are in flight together (each is a cache round trip)
-        for (int w0 = 0; w0 < words; w0 += 4) {
-            float pa[4], pb[4];
-            uint64_t mword = 0;
+    // ---- phase 1: bitmaps.  Item = (64-k word, block of BT x BT tiles); two items per step so
+    // that their norm loads are in flight together (each is a cache round trip).  Loads are
+    // unconditional from clamped addresses; what lies outside the matrix is masked after the
+    // ballot (k per lane, tile rows / columns per wave).
+    struct Item {
+        float pa[BT], pb[BT];
+    };
+    auto load_item = [&](int item, Item &it) {
+        const int q = item % G::NQ, w = item / G::NQ;
+        const int k = w * 64 + lane;
+        const int kc = k < nbK ? k : nbK - 1;
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int k = (w0 + u) * 64 + lane;
-                const bool live = inside && k < nbK;
-                pa[u] = live ? ra[k] : 0.0f;
-                pb[u] = live ? rb[k] : 0.0f;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int w = w0 + u;
-                if (w >= words) break;
-                const int k = w * 64 + lane;
-                bool keep = false;
-                if (inside && k < nbK) {
-                    const float p = pa[u] * pb[u];
-                    keep = p >= tau;
-                }
-                const uint64_t m = __ballot(keep);
-                if (keep) {
-                    const int pos = base + __builtin_popcountll(m & ((1ull << lane) - 1ull));
-                    g.klist[tid * nbK + pos] = (uint16_t)k;
-                }
-                base += __builtin_popcountll(m);
-                if (lane == u) mword = m;              // lane u keeps word w0 + u
-            }
-            // one store of up to four words per step instead of one per word
-            if (lane < 4 && w0 + lane < words) {
-                lmask[(size_t)t * words + w0 + lane] = mword;
-                if (inside) g.mask[tid * words + w0 + lane] = mword;
-            }
+        for (int a = 0; a < BT; a++) {
+            const int i = mi * MT + (q / G::QD) * BT + a;
+            it.pa[a] = g.nA[(int64_t)(i < nbM ? i : nbM - 1) * nbK + kc];
         }
-        if (inside && lane == 0) g.counts[tid] = base;
-        my_work += base;
+#pragma unroll
+        for (int b = 0; b < BT; b++) {
+            const int j = mj * MT + (q % G::QD) * BT + b;
+            it.pb[b] = g.nBt[(int64_t)(j < nbN ? j : nbN - 1) * nbK + kc];
+        }
+    };
+    // whole macro tile inside the matrix: only the last k word may need masking
+    const bool interior = (mi + 1) * MT <= nbM && (mj + 1) * MT <= nbN;
+    auto gate_item = [&](int item, const Item &it) {
+        const int q = item % G::NQ, w = item / G::NQ;
+        const int ti0 = (q / G::QD) * BT, tj0 = (q % G::QD) * BT;
+        int mlo = 0, mhi = 0;                 // lane a*BT+b collects the word of tile (a, b)
+        if (interior && (w + 1) * 64 <= nbK) {
+#pragma unroll
+            for (int a = 0; a < BT; a++)
+#pragma unroll
+                for (int b = 0; b < BT; b++) {
+                    const uint64_t m = __ballot(it.pa[a] * it.pb[b] >= tau);
+                    set_lane(mlo, (uint32_t)m, a * BT + b);
+                    set_lane(mhi, (uint32_t)(m >> 32), a * BT + b);
+                }
+        } else {
+            const uint64_t kmask = __ballot(w * 64 + lane < nbK);
+#pragma unroll
+            for (int a = 0; a < BT; a++)
+#pragma unroll
+                for (int b = 0; b < BT; b++) {
+                    // wave-uniform all-ones / zero: is tile (a, b) of the block inside the matrix
+                    const uint64_t inside =
+                        0ull - (uint64_t)((mi * MT + ti0 + a < nbM) & (mj * MT + tj0 + b < nbN));
+                    const uint64_t m = __ballot(it.pa[a] * it.pb[b] >= tau) & kmask & inside;
+                    set_lane(mlo, (uint32_t)m, a * BT + b);
+                    set_lane(mhi, (uint32_t)(m >> 32), a * BT + b);
+                }
+        }
+        if (lane < BT * BT)
+            lmask[(size_t)w * NTP + (ti0 + lane / BT) * MT + tj0 + lane % BT] =
+                ((uint64_t)(uint32_t)mhi << 32) | (uint32_t)mlo;
+    };
+    const int n_items = G::NQ * words;
+    for (int it0 = wave; it0 < n_items; it0 += 8) {
+        const int it1 = it0 + 4;
+        Item i0, i1;
+        load_item(it0, i0);
+        if (it1 < n_items) load_item(it1, i1);
+        gate_item(it0, i0);
+        if (it1 < n_items) gate_item(it1, i1);
     }
-    if (lane == 0) atomicAdd(&s_work, my_work);
     __syncthreads();
 
-    // ---- phase 2: union list with per-tile bits.  Entries whose k is kept by
-    // every tile of the macro tile ("full") come first, then the partial ones,
-    // each group in ascending k: the GEMM runs a branch-free loop over the
-    // first group.
-    int *wfull = wsum;                       // [words + 1] prefix of full entries
-    int *wpart = wsum + (words + 1);         // [words + 1] prefix of partial entries
-    for (int w = threadIdx.x; w < words; w += 256) {
-        uint64_t u = 0, f = ~0ull;
-        for (int t = 0; t < NT; t++) {
-            const uint64_t m = lmask[(size_t)t * words + w];
-            u |= m;
-            f &= m;
+    // ---- phase 2a: per-tile counts, the macro tile's kept-product total, bitmaps to memory
+    int work = 0;
+    if (wave == 0) {
+        int cnt = 0;
+        if (lane < NT) {
+            for (int w = 0; w < words; w++) cnt += __builtin_popcountll(lmask[(size_t)w * NTP + lane]);
+            const int i = mi * MT + lane / MT, j = mj * MT + lane % MT;
+            if (i < nbM && j < nbN) g.counts[(int64_t)i * nbN + j] = cnt;
         }
-        wfull[w + 1] = __builtin_popcountll(f);
-        wpart[w + 1] = __builtin_popcountll(u & ~f);
+        work = cnt;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) work += __shfl_xor(work, off, 64);
+    }
+    const float inv_words = 1.0f / (float)words;     // e < 2^16, words <= 1024: the quotient below is exact
+    for (int e = threadIdx.x; e < NT * words; e += 256) {
+        const int t = (int)(((float)e + 0.5f) * inv_words), w = e - t * words;
+        const int i = mi * MT + t / MT, j = mj * MT + t % MT;
+        if (i < nbM && j < nbN) g.mask[((int64_t)i * nbN + j) * words + w] = lmask[(size_t)w * NTP + t];
+    }
+    __syncthreads();
+
+    // ---- phase 2b: transpose every word in place: entry b of word w becomes the set of tiles
+    // (bit t = tile t of the macro tile) that keep k = 64 w + b, NTP bits wide
+    auto tile_bits = [&](int w, int b) -> uint64_t {
+        if constexpr (NTP == 64) return lmask[(size_t)w * 64 + b];
+        else if constexpr (NTP == 16) return reinterpret_cast<const uint16_t *>(lmask + (size_t)w * 16)[b];
+        else return reinterpret_cast<const uint8_t *>(lmask + (size_t)w * 8)[b];
+    };
+    for (int w = wave; w < words; w += 4) {
+        const uint64_t row = lane < NT ? lmask[(size_t)w * NTP + lane] : 0ull;
+        const uint64_t bits = transpose64(row, lane);
+        const uint64_t u = __ballot(bits != 0ull), f = __ballot(bits == G::FULL);
+        // the wave has read all rows of the word before any lane writes its column
+        if constexpr (NTP == 64) lmask[(size_t)w * 64 + lane] = bits;
+        else if constexpr (NTP == 16) reinterpret_cast<uint16_t *>(lmask + (size_t)w * 16)[lane] = (uint16_t)bits;
+        else reinterpret_cast<uint8_t *>(lmask + (size_t)w * 8)[lane] = (uint8_t)bits;
+        if (lane == 0) {
+            luf[2 * w] = u;
+            luf[2 * w + 1] = f;
+            wfull[w + 1] = __builtin_popcountll(f);
+            wpart[w + 1] = __builtin_popcountll(u & ~f);
+        }
     }
     if (threadIdx.x == 0) { wfull[0] = 0; wpart[0] = 0; }
     __syncthreads();
-    // inclusive scans over words (Hillis-Steele in LDS; words is small)
-    for (int off = 1; off <= words; off <<= 1) {
-        int addf[5], addp[5];        // words <= 1024: at most 5 per thread
-        int n = 0;
-        for (int w = threadIdx.x; w <= words; w += 256) {
-            addf[n] = w >= off ? wfull[w - off] : 0;
-            addp[n] = w >= off ? wpart[w - off] : 0;
-            n++;
+
+    // ---- phase 2c: union list with per-tile bits.  Entries whose k is kept by
+    // every tile of the macro tile ("full") come first, then the partial ones,
+    // each group in ascending k: the GEMM runs a branch-free loop over the
+    // first group.  Inclusive scans over the words give each word's offset.
+    if (words < 64) {
+        if (wave == 0) {
+            int vf = lane <= words ? wfull[lane] : 0, vp = lane <= words ? wpart[lane] : 0;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int tf = __shfl_up(vf, off, 64), tp = __shfl_up(vp, off, 64);
+                if (lane >= off) { vf += tf; vp += tp; }
+            }
+            if (lane <= words) { wfull[lane] = vf; wpart[lane] = vp; }
         }
         __syncthreads();
-        n = 0;
-        for (int w = threadIdx.x; w <= words; w += 256) {
-            wfull[w] += addf[n];
-            wpart[w] += addp[n];
-            n++;
+    } else {
+        // Hillis-Steele in LDS
+        for (int off = 1; off <= words; off <<= 1) {
+            int addf[5], addp[5];        // words <= 1024: at most 5 per thread
+            int n = 0;
+            for (int w = threadIdx.x; w <= words; w += 256) {
+                addf[n] = w >= off ? wfull[w - off] : 0;
+                addp[n] = w >= off ? wpart[w - off] : 0;
+                n++;
+            }
+            __syncthreads();
+            n = 0;
+            for (int w = threadIdx.x; w <= words; w += 256) {
+                wfull[w] += addf[n];
+                wpart[w] += addp[n];
+                n++;
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
     const int n_full = wfull[words];
     const int n_part = wpart[words];
@@ -129,37 +229,26 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     // them on the same A row panels and B column panels at the same time.
     int rot_f = 0, rot_p = 0;              // entries of each group below the anchor
     {
-        const int mMT = nMacN > 0 ? MT : MT;
         const int sm = mi / SUPER_M, sn = mj / SUPER_N;
-        const float ic = ((sm * SUPER_M + 0.5f * SUPER_M) * mMT) / (float)nbM;
-        const float jc = ((sn * SUPER_N + 0.5f * SUPER_N) * mMT) / (float)nbN;
-        float fa = 0.5f * (ic + jc) * (float)nbK - 0.5f * SUPER_N * mMT;
+        const float ic = ((sm * SUPER_M + 0.5f * SUPER_M) * MT) / (float)nbM;
+        const float jc = ((sn * SUPER_N + 0.5f * SUPER_N) * MT) / (float)nbN;
+        const float fa = 0.5f * (ic + jc) * (float)nbK - 0.5f * SUPER_N * MT;
         int anchor = (int)fa;
         anchor = anchor < 0 ? 0 : (anchor > nbK - 1 ? nbK - 1 : anchor);
         const int wa = anchor >> 6, ba = anchor & 63;
-        uint64_t u = 0, f = ~0ull;
-        for (int t = 0; t < NT; t++) {
-            const uint64_t m = lmask[(size_t)t * words + wa];
-            u |= m;
-            f &= m;
-        }
+        const uint64_t u = luf[2 * wa], f = luf[2 * wa + 1];
         const uint64_t below = (1ull << ba) - 1ull;
         rot_f = wfull[wa] + __builtin_popcountll(f & below);
         rot_p = wpart[wa] + __builtin_popcountll(u & ~f & below);
     }
     for (int k = threadIdx.x; k < nbK; k += 256) {
         const int w = k >> 6, b = k & 63;
-        uint64_t u = 0, f = ~0ull, bits = 0;
-        for (int t = 0; t < NT; t++) {
-            const uint64_t m = lmask[(size_t)t * words + w];
-            u |= m;
-            f &= m;
-            bits |= ((m >> b) & 1ull) << t;
-        }
-        if ((u >> b) & 1ull) {
+        const uint64_t bits = tile_bits(w, b);
+        if (bits != 0ull) {
+            const uint64_t u = luf[2 * w], f = luf[2 * w + 1];
             const uint64_t below = (1ull << b) - 1ull;
             int pos;
-            if ((f >> b) & 1ull) {
+            if (bits == G::FULL) {
                 pos = wfull[w] + __builtin_popcountll(f & below) - rot_f;
                 if (pos < 0) pos += n_full;
             } else {
@@ -168,6 +257,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
                 pos += n_full;
             }
             uint32_t need = 0;
+#pragma unroll
             for (int a = 0; a < MT; a++) {
                 const uint32_t rowbits = (uint32_t)(bits >> (a * MT)) & ((1u << MT) - 1u);
                 if (rowbits) need |= 1u << a;
@@ -184,7 +274,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     if (threadIdx.x == 0) {
         g.macro_count[2 * macro] = n_full + n_part;
         g.macro_count[2 * macro + 1] = n_full;
-        g.macro_work[macro] = s_work;
+        g.macro_work[macro] = work;
     }
 }
 
@@ -334,15 +424,43 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;
 }
 
+// Per-tile ascending list of kept k (the reference's offset[], cuSpAMM.cu:315-325)
+// from the gate's bitmaps: one wave per output tile, popcount below the lane's
+// bit gives every kept k its slot.
+__global__ __launch_bounds__(256) void k_klist(const uint64_t *__restrict__ mask, uint16_t *__restrict__ klist,
+                                               int64_t n_tiles, int nbK, int words) {
+    const int lane = threadIdx.x & 63;
+    const int64_t tid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tid >= n_tiles) return;
+    int base = 0;
+    for (int w = 0; w < words; w++) {
+        const uint64_t m = mask[tid * words + w];
+        if ((m >> lane) & 1ull)
+            klist[tid * nbK + base + __builtin_popcountll(m & ((1ull << lane) - 1ull))] = (uint16_t)(w * 64 + lane);
+        base += __builtin_popcountll(m);
+    }
+}
+
+hipError_t launch_klist(const uint64_t *mask, uint16_t *klist, int64_t n_tiles, int64_t nbK, hipStream_t s) {
+    k_klist<<<(unsigned)((n_tiles + 3) / 4), 256, 0, s>>>(mask, klist, n_tiles, (int)nbK, (int)((nbK + 63) / 64));
+    return hipGetLastError();
+}
+
 size_t gate_lds_bytes(int tile, int64_t nbK) {
     const int MT = macro_dim(tile);
+    const size_t ntp = MT * MT < 8 ? 8 : MT * MT;
     const size_t words = (size_t)((nbK + 63) / 64);
-    return (size_t)MT * MT * words * 8 + 2 * (words + 1) * 4 + 8;
+    return ntp * words * 8 + words * 16 + 2 * (words + 1) * 4;
 }
 
 // k_gate may use all of a CU's LDS for the macro tile's bitmaps (its workgroups are short)
 hipError_t gate_init() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate), hipFuncAttributeMaxDynamicSharedMemorySize,
+    hipError_t e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)gate_lds_limit())) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<4>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)gate_lds_limit())) != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)gate_lds_limit());
 }
 
@@ -352,7 +470,12 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     const int nMacM = (int)((nbM + MT - 1) / MT), nMacN = (int)((nbN + MT - 1) / MT);
     const int n_macro = nMacM * nMacN;
     const size_t lds = gate_lds_bytes(tile, nbK);
-    k_gate<<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, MT, nMacN, tau);
+    switch (MT) {
+        case 8: k_gate<8><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
+        case 4: k_gate<4><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
+        case 2: k_gate<2><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
+        default: return hipErrorInvalidValue;
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;

@@ -93,7 +93,6 @@ GateBuffers gate_buffers(spamm_ctx *c) {
     g.nA = (const float *)c->nA.p;
     g.nBt = (const float *)c->nBt.p;
     g.counts = (int32_t *)c->counts.p;
-    g.klist = (uint16_t *)c->klist.p;
     g.mask = (uint64_t *)c->mask.p;
     g.macro_list = (MacroEntry *)c->macro_list.p;
     g.macro_count = (int32_t *)c->macro_count.p;
@@ -280,10 +279,9 @@ int spamm_gate(spamm_ctx *c, float tau) {
     int rc = set_device(c);
     if (rc) return rc;
     const Shape s = shape_of(c);
-    if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // K / tile beyond ~20 000 (tile 32)
+    if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // K / tile beyond ~19 500 (tile 32)
     const size_t nt = (size_t)s.nbM * s.nbN;
     if ((rc = ensure(c, c->counts, nt * 4))) return rc;
-    if ((rc = ensure(c, c->klist, nt * s.nbK * 2))) return rc;
     if ((rc = ensure(c, c->mask, nt * s.words * 8))) return rc;
     if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
     if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
@@ -655,7 +653,13 @@ int spamm_get_klist(spamm_ctx *c, uint16_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
     if (!c->have_gate) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
-    return copy_out(c, c->klist.p, host_out, (size_t)s.nbM * s.nbN * s.nbK * 2);
+    // built from the bitmaps on demand: the multiply itself never reads per-tile lists
+    int rc = set_device(c);
+    if (rc) return rc;
+    const size_t bytes = (size_t)s.nbM * s.nbN * s.nbK * 2;
+    if ((rc = ensure(c, c->klist, bytes))) return rc;
+    HIPCHK(c, launch_klist((const uint64_t *)c->mask.p, (uint16_t *)c->klist.p, s.nbM * s.nbN, s.nbK, c->stream));
+    return copy_out(c, c->klist.p, host_out, bytes);
 }
 
 int spamm_get_mask(spamm_ctx *c, uint64_t *host_out) {

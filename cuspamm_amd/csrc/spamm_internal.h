@@ -55,7 +55,6 @@ struct GateBuffers {
     const float *nA;        // [nbM x nbK]
     const float *nBt;       // [nbN x nbK]  (transposed B norm map)
     int32_t *counts;        // [nbM*nbN]
-    uint16_t *klist;        // [nbM*nbN*nbK]
     uint64_t *mask;         // [nbM*nbN*words]
     MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
     int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
@@ -93,6 +92,8 @@ inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k
 hipError_t gate_init();   // one-time kernel attribute set-up
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
                        float tau, hipStream_t s);
+// per-tile ascending k lists [n_tiles x nbK] from the gate's bitmaps (read-back only)
+hipError_t launch_klist(const uint64_t *mask, uint16_t *klist, int64_t n_tiles, int64_t nbK, hipStream_t s);
 
 // tau selection (kernels_tau.hip)
 struct TauState {
