@@ -286,45 +286,38 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 //      the XCDs in snake order: every XCD owns whole super tiles, so the
 //      workgroups sharing one L2 share A row panels and B column panels, and
 //      the XCDs get equal work.
-//   2. Inside an XCD the macro tiles are ordered by work level (SCHED_LEVELS
-//      classes of the kept-product count, heaviest first) and, inside a
-//      level, in super-tile order.  With two levels (computing / nothing
-//      kept) the computing macro tiles simply run super tile by super tile:
-//      measured on banded inputs, finer heaviest-first classes did not
-//      shorten the tail but pulled neighbours apart (10 % more L2 misses).
+//   2. Inside an XCD the computing macro tiles run super tile by super tile
+//      (measured on banded inputs, heaviest-first classes inside an XCD did
+//      not shorten the tail but pulled neighbours apart: 10 % more L2 misses).
 //   3. Macro tiles with nothing kept come last in each XCD's sequence: their
 //      workgroups only write zeros and start when CUs fall idle at the end.
-// Output: order[x * P + q] = macro tile id of XCD x's q-th workgroup,
-// sched[x] = number of computing items, sched[8 + x] = number of all items.
+// Output: order[x * P + q] = macro tile id of XCD x's q-th workgroup for
+// q < sched[8 + x] (entries beyond are not written), sched[x] = number of
+// computing items, sched[8 + x] = number of all items.
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
                                                 int n_super, int rounds) {
-    extern __shared__ int swork[];               // [n_super] work, then reused: [n_super] id by rank
+    extern __shared__ int swork[];               // [n_super] work, then [n_super] super tile id by rank
     int *srank_id = swork + n_super;
     __shared__ unsigned long long total;
-    __shared__ int maxwork;
     const int P = rounds * SUPER_M * SUPER_N;
-    if (threadIdx.x == 0) { total = 0; maxwork = 1; }
+    if (threadIdx.x == 0) total = 0;
     __syncthreads();
     unsigned long long mine = 0;
-    int mymax = 0;
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int sm = sid / nSupN, sn = sid % nSupN;
         int w = 0;
+#pragma unroll
         for (int a = 0; a < SUPER_M; a++)
+#pragma unroll
             for (int b = 0; b < SUPER_N; b++) {
                 const int mi = sm * SUPER_M + a, mj = sn * SUPER_N + b;
-                if (mi < nMacM && mj < nMacN) {
-                    const int mw = g.macro_work[mi * nMacN + mj];
-                    w += mw;
-                    mymax = mw > mymax ? mw : mymax;
-                }
+                if (mi < nMacM && mj < nMacN) w += g.macro_work[mi * nMacN + mj];
             }
         swork[sid] = w;
         mine += (unsigned long long)w;
     }
-    atomicAdd(&total, mine);
-    atomicMax(&maxwork, mymax);
+    if (mine) atomicAdd(&total, mine);
     __syncthreads();
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int w = swork[sid];
@@ -335,90 +328,47 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         }
         srank_id[rank] = sid;
     }
-    for (int i = threadIdx.x; i < NUM_XCD * P; i += blockDim.x) g.order[i] = -1;
     __syncthreads();
 
-    // item of XCD x at raw position p (round-major, then slot), or -1; level of that item
-    const int mw_max = maxwork;
-    auto item_at = [&](int x, int p, int &level) -> int {
+    // macro tile of XCD x at raw position p (round-major, then slot inside the super tile), or -1
+    auto macro_at = [&](int x, int p) -> int {
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
         const int sr = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - x : x);
-        if (sr >= n_super) return -1;
+        if (p >= P || sr >= n_super) return -1;
         const int sid = srank_id[sr];
         const int mi = (sid / nSupN) * SUPER_M + slot / SUPER_N, mj = (sid % nSupN) * SUPER_N + slot % SUPER_N;
-        if (mi >= nMacM || mj >= nMacN) return -1;
-        const int m = mi * nMacN + mj;
-        const int mw = g.macro_work[m];
-        level = mw > 0 ? 1 + (int)(((int64_t)(mw - 1) * (SCHED_LEVELS - 1)) / mw_max) : 0;
-        return m;
+        return (mi < nMacM && mj < nMacN) ? mi * nMacN + mj : -1;
     };
-    // raw sequence (round-major, slot-minor) with the level in the top byte, in the upper half of `order`
-    int32_t *raw = g.order + NUM_XCD * P;
-    for (int i = threadIdx.x; i < NUM_XCD * P; i += blockDim.x) {
-        int level = 0;
-        const int m = item_at(i / P, i % P, level);
-        raw[i] = m >= 0 ? (m | (level << 24)) : -1;
-    }
-    __syncthreads();
-    // one wave per XCD: count per level, prefix (heaviest level first, empty tiles last), stable scatter
+    // one wave per XCD: computing macro tiles to the front in raw order, empty ones from the back
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (wave < NUM_XCD) {
         const int x = wave;
-        const int32_t *rx = raw + x * P;
-        int mycnt = 0;                       // lane lv < SCHED_LEVELS keeps the count of level lv
+        int nall = 0;                            // macro tiles in this XCD's sequence (no memory access)
+        for (int p0 = 0; p0 < P; p0 += 64) nall += __builtin_popcountll(__ballot(macro_at(x, p0 + lane) >= 0));
+        int nc = 0, ne = 0;
+        const uint64_t below = (1ull << lane) - 1ull;
         // (loads of UN chunks are issued together: the wave is alone here and each one is an L2 round trip)
         constexpr int UN = 8;
         for (int p0 = 0; p0 < P; p0 += 64 * UN) {
-            int vv[UN];
+            int mm[UN], ww[UN];
 #pragma unroll
             for (int u = 0; u < UN; u++) {
-                const int p = p0 + u * 64 + lane;
-                vv[u] = p < P ? rx[p] : -1;
+                mm[u] = macro_at(x, p0 + u * 64 + lane);
+                ww[u] = mm[u] >= 0 ? g.macro_work[mm[u]] : 0;
             }
 #pragma unroll
             for (int u = 0; u < UN; u++) {
-                const int level = vv[u] >= 0 ? (vv[u] >> 24) : -1;
-#pragma unroll
-                for (int lv = 0; lv < SCHED_LEVELS; lv++) {
-                    const int c = __builtin_popcountll(__ballot(level == lv));
-                    if (lane == lv) mycnt += c;
-                }
+                const bool comp = mm[u] >= 0 && ww[u] > 0, empty = mm[u] >= 0 && ww[u] <= 0;
+                const uint64_t bc = __ballot(comp), be = __ballot(empty);
+                if (comp) g.order[x * P + nc + __builtin_popcountll(bc & below)] = mm[u];
+                if (empty) g.order[x * P + nall - 1 - (ne + __builtin_popcountll(be & below))] = mm[u];
+                nc += __builtin_popcountll(bc);
+                ne += __builtin_popcountll(be);
             }
-        }
-        // exclusive prefix over levels in descending order: base(lv) = sum of counts of levels > lv
-        int base = 0, ncomp = 0, nall = 0;
-#pragma unroll
-        for (int lv = SCHED_LEVELS - 1; lv >= 0; lv--) {
-            const int c = __shfl(mycnt, lv, 64);
-            if (lane == lv) base = nall;
-            if (lv == 0) ncomp = nall;
-            nall += c;
         }
         if (lane == 0) {
-            g.sched[x] = ncomp;
+            g.sched[x] = nc;
             g.sched[NUM_XCD + x] = nall;
-        }
-        for (int p0 = 0; p0 < P; p0 += 64 * UN) {
-            int vv[UN];
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-                const int p = p0 + u * 64 + lane;
-                vv[u] = p < P ? rx[p] : -1;
-            }
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-                const int v = vv[u];
-                const int level = v >= 0 ? (v >> 24) : -1;
-                int pos = -1;
-#pragma unroll
-                for (int lv = 0; lv < SCHED_LEVELS; lv++) {
-                    const uint64_t bal = __ballot(level == lv);
-                    const int b0 = __shfl(base, lv, 64);
-                    if (level == lv) pos = b0 + __builtin_popcountll(bal & ((1ull << lane) - 1ull));
-                    if (lane == lv) base += __builtin_popcountll(bal);
-                }
-                if (pos >= 0) g.order[x * P + pos] = v & 0xffffff;
-            }
         }
     }
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;

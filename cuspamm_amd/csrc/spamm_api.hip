@@ -286,7 +286,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
     if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
     if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
-    if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * NUM_XCD * SUPER_M * SUPER_N * 2 * 4))) return rc;
+    if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * NUM_XCD * SUPER_M * SUPER_N * 4))) return rc;
     if ((rc = ensure(c, c->sched, 2 * NUM_XCD * 4))) return rc;
     if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));

@@ -30,7 +30,6 @@ inline int macro_dim(int tile) { return 256 / tile; }
 constexpr int SUPER_M = 4;
 constexpr int SUPER_N = 8;
 constexpr int NUM_XCD = 8;
-constexpr int SCHED_LEVELS = 2;   // work classes used to order macro tiles inside an XCD (0 = nothing kept)
 
 // Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin.
 inline int sched_rounds(int tile, int64_t nbM, int64_t nbN) {
@@ -59,7 +58,7 @@ struct GateBuffers {
     MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
     int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
     int32_t *macro_work;    // [n_macro]       kept products in the macro tile
-    int32_t *order;         // [2][8 * P]      macro tile of XCD x's q-th workgroup (P = rounds * 32), -1 = none; second half is scratch
+    int32_t *order;         // [8 * P]         macro tile of XCD x's q-th workgroup (P = rounds * 32), valid for q < sched[8 + x]
     int32_t *sched;         // [16]            per XCD: computing items, all items
     int64_t *kept_total;    // [1]  kept products
 };
