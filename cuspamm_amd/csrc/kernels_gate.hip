@@ -297,24 +297,25 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
                                                 int n_super, int rounds) {
-    extern __shared__ int swork[];               // [n_super] work, then [n_super] super tile id by rank
+    extern __shared__ int swork[];               // [n_super] work, then [n_super] super tile origin by rank
     int *srank_id = swork + n_super;
     __shared__ unsigned long long total;
     const int P = rounds * SUPER_M * SUPER_N;
     if (threadIdx.x == 0) total = 0;
+    // (this kernel is one workgroup on an idle GPU: its run time is memory round trips and
+    // instruction fetch, so every thread takes one macro tile row of one super tile -- all loads
+    // of the kernel's first step are in flight at once -- and the code is kept small)
+    for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) swork[sid] = 0;
     __syncthreads();
     unsigned long long mine = 0;
-    for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
-        const int sm = sid / nSupN, sn = sid % nSupN;
+    for (int e = threadIdx.x; e < n_super * SUPER_M; e += blockDim.x) {
+        const int sid = e / SUPER_M, a = e % SUPER_M;
+        const int mi = (sid / nSupN) * SUPER_M + a, mj0 = (sid % nSupN) * SUPER_N;
         int w = 0;
 #pragma unroll
-        for (int a = 0; a < SUPER_M; a++)
-#pragma unroll
-            for (int b = 0; b < SUPER_N; b++) {
-                const int mi = sm * SUPER_M + a, mj = sn * SUPER_N + b;
-                if (mi < nMacM && mj < nMacN) w += g.macro_work[mi * nMacN + mj];
-            }
-        swork[sid] = w;
+        for (int b = 0; b < SUPER_N; b++)
+            if (mi < nMacM && mj0 + b < nMacN) w += g.macro_work[mi * nMacN + mj0 + b];
+        if (w) atomicAdd(&swork[sid], w);
         mine += (unsigned long long)w;
     }
     if (mine) atomicAdd(&total, mine);
@@ -326,7 +327,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
             const int wj = swork[j];
             rank += (wj > w) || (wj == w && j < sid);
         }
-        srank_id[rank] = sid;
+        srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
     }
     __syncthreads();
 
@@ -335,8 +336,8 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
         const int sr = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - x : x);
         if (p >= P || sr >= n_super) return -1;
-        const int sid = srank_id[sr];
-        const int mi = (sid / nSupN) * SUPER_M + slot / SUPER_N, mj = (sid % nSupN) * SUPER_N + slot % SUPER_N;
+        const int origin = srank_id[sr];
+        const int mi = (origin >> 16) + slot / SUPER_N, mj = (origin & 0xffff) + slot % SUPER_N;
         return (mi < nMacM && mj < nMacN) ? mi * nMacN + mj : -1;
     };
     // one wave per XCD: computing macro tiles to the front in raw order, empty ones from the back
