@@ -59,7 +59,8 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT, uint4 *__restrict__ packed2,
-                                                 float *__restrict__ nm2) {
+                                                 float *__restrict__ nm2, const float *__restrict__ rowmax,
+                                                 float tau_skip) {
     constexpr int TPS = SW / B;           // tiles per strip
     constexpr int LPR = SW / 4;           // lanes across one strip row
     constexpr int RH = 64 / LPR;          // strip rows per wave-wide load
@@ -162,23 +163,30 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             }
         }
     };
-    // packed tiles out (256 threads x 16 bytes = 4 KiB per step, contiguous per tile) and norms
-    // (one wave per tile, canonical order)
-    auto emit = [&](bool as_b, uint4 *__restrict__ pk, float *__restrict__ nmo, float *__restrict__ nmTo) {
+    // packed tiles out (256 threads x 16 bytes = 4 KiB per step, contiguous per tile)
+    __shared__ int s_skip[TPS];
+    auto copy_out = [&](bool as_b, uint4 *__restrict__ pk, bool prune) {
 #pragma unroll
         for (int i = 0; i < TPS * VPT / 256; i++) {
             const int vi = threadIdx.x + 256 * i;
             const int tt = vi / VPT, iv = vi % VPT;
             const int64_t Jt = sc * TPS + tt;
-            if (Jt < nbc) {
+            if (Jt < nbc && !(prune && s_skip[tt])) {
                 const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
                 const int64_t tile = as_b ? Jt * nbr + I : I * nbc + Jt;
                 __builtin_nontemporal_store(*reinterpret_cast<const u32x4n *>(&d), reinterpret_cast<u32x4n *>(pk + tile * VPT + iv));
             }
         }
+    };
+    // norms: one wave per tile, canonical order.  With `prune` (A role, tau known, B's norm map
+    // done) the wave also decides whether any product can keep the tile: fl(nA[i,k] * nB[k,j]) <=
+    // fl(nA[i,k] * max_j nB[k,j]) because rounding is monotone, so a tile whose product with the
+    // row maximum is below tau is never read by the GEMM and its fp16 copy need not be written.
+    auto norms = [&](bool as_b, float *__restrict__ nmo, float *__restrict__ nmTo, bool prune) {
         for (int tt = wave; tt < TPS; tt += 4) {
             const int64_t Jt = sc * TPS + tt;
             if (Jt >= nbc) break;
+            const float rmax = prune ? rowmax[Jt] : 0.0f;
             float partial = 0.0f;
 #pragma unroll
             for (int it = 0; it < STEPS; it++) {
@@ -190,13 +198,24 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
                 const float nv = sqrtf(partial);
                 nmo[I * nbc + Jt] = nv;
                 if (as_b) nmTo[Jt * nbr + I] = nv;
+                if (prune) s_skip[tt] = nv * rmax < tau_skip;
             }
         }
+    };
+    auto emit = [&](bool as_b, uint4 *__restrict__ pk, float *__restrict__ nmo, float *__restrict__ nmTo) {
+        copy_out(as_b, pk, false);
+        norms(as_b, nmo, nmTo, false);
     };
     if (ROLE == 0) {
         stage_a();
         __syncthreads();
-        emit(false, packed, nm, nullptr);
+        if (rowmax != nullptr) {
+            norms(false, nm, nullptr, true);
+            __syncthreads();
+            copy_out(false, packed, true);
+        } else {
+            emit(false, packed, nm, nullptr);
+        }
     } else if (ROLE == 1) {
         stage_b();
         __syncthreads();
@@ -210,6 +229,20 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
         __syncthreads();
         emit(true, packed2, nm2, nmT);
     }
+}
+
+// rowmax[k] = max_j nB[k, j] (nB row-major [nbK x nbN]); one wave per row.  NaNs are ignored:
+// a NaN product is never kept.
+__global__ __launch_bounds__(256) void k_rowmax(const float *__restrict__ nB, int64_t nbK, int64_t nbN,
+                                                float *__restrict__ rowmax) {
+    const int lane = threadIdx.x & 63;
+    const int64_t k = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (k >= nbK) return;
+    float m = 0.0f;
+    for (int64_t j = lane; j < nbN; j += 64) m = fmaxf(m, nB[k * nbN + j]);
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) m = fmaxf(m, __shfl_xor(m, s, 64));
+    if (lane == 0) rowmax[k] = m;
 }
 
 // ------------------------------------------------------------- utilities
@@ -283,24 +316,30 @@ __global__ __launch_bounds__(256) void k_fill_decay(float *__restrict__ X, int64
 // ---------------------------------------------------------------- launchers
 template <int ROLE, bool IN16>
 static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int tile, void *packed, float *nm,
-                                 float *nmT, hipStream_t s, void *packed2 = nullptr, float *nm2 = nullptr) {
+                                 float *nmT, hipStream_t s, void *packed2 = nullptr, float *nm2 = nullptr,
+                                 const float *rowmax = nullptr, float tau_skip = 0.0f) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
     const int sw = tile == 128 ? 128 : 256;
     const int64_t nstrip = (cols + sw - 1) / sw;
     const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
-        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
-        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
-        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2); break;
+        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
 hipError_t launch_normmap_a(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
-                            float *nm, hipStream_t s) {
-    return in16 ? launch_normmap<0, true>(X, rows, cols, tile, packed, nm, nullptr, s)
-                : launch_normmap<0, false>(X, rows, cols, tile, packed, nm, nullptr, s);
+                            float *nm, const float *rowmax, float tau_skip, hipStream_t s) {
+    return in16 ? launch_normmap<0, true>(X, rows, cols, tile, packed, nm, nullptr, s, nullptr, nullptr, rowmax, tau_skip)
+                : launch_normmap<0, false>(X, rows, cols, tile, packed, nm, nullptr, s, nullptr, nullptr, rowmax, tau_skip);
+}
+
+hipError_t launch_rowmax(const float *nB, int64_t nbK, int64_t nbN, float *rowmax, hipStream_t s) {
+    k_rowmax<<<(unsigned)((nbK + 3) / 4), 256, 0, s>>>(nB, nbK, nbN, rowmax);
+    return hipGetLastError();
 }
 
 hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void *packedA, float *nmA,

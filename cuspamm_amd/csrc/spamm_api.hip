@@ -34,8 +34,12 @@ struct spamm_ctx {
     int tile = 0;
     bool have_a = false, have_b = false, have_gate = false;
     float tau = 0.0f;
+    // A's fp16 copy was written by a tau-aware pass: tiles that no product can keep at
+    // a_pruned_tau are missing, so the copy serves a GEMM only for tau >= a_pruned_tau
+    bool a_pruned = false;
+    float a_pruned_tau = 0.0f;
 
-    DevBuf packedA, packedB, nA, nB, nBt;
+    DevBuf packedA, packedB, nA, nB, nBt, rowmaxB;
     DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, sched, kept_total;
     DevBuf scratch;   // read-back staging / decay table
     DevBuf tauws;     // tau selection workspace
@@ -114,6 +118,7 @@ void reset_shape(spamm_ctx *c, int tile) {
     c->tile = tile;
     c->M = c->K = c->N = 0;
     c->have_a = c->have_b = c->have_gate = false;
+    c->a_pruned = false;
 }
 
 int copy_out(spamm_ctx *c, const void *dev, void *host, size_t bytes) {
@@ -174,7 +179,7 @@ int spamm_destroy(spamm_ctx *c) {
     if (!c) return SPAMM_EINVAL;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->counts, &c->klist,
+    DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->rowmaxB, &c->counts, &c->klist,
                       &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
                       &c->sched, &c->kept_total, &c->scratch, &c->tauws};
     for (DevBuf *b : bufs)
@@ -201,7 +206,7 @@ int spamm_synchronize(spamm_ctx *c) {
 }
 
 static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_t rows, int64_t cols,
-                       int32_t tile) {
+                       int32_t tile, const float *prune_tau = nullptr) {
     if (!c || !dX || !tile_ok(tile)) return SPAMM_EINVAL;
     if (role != SPAMM_ROLE_A && role != SPAMM_ROLE_B) return SPAMM_EINVAL;
     if (rows <= 0 || cols <= 0 || rows % tile || cols % tile) return SPAMM_EINVAL;
@@ -217,12 +222,22 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
         c->K = cols;
         if ((rc = ensure(c, c->packedA, (size_t)rows * cols * 2))) return rc;
         if ((rc = ensure(c, c->nA, nt * 4))) return rc;
+        // tau-aware pass: needs B's norm map of the same K (the caller checked have_b)
+        const bool prune = prune_tau != nullptr && c->have_b && c->nB.p;
+        if (prune) {
+            if ((rc = ensure(c, c->rowmaxB, (size_t)(cols / tile) * 4))) return rc;
+            HIPCHK(c, launch_rowmax((const float *)c->nB.p, cols / tile, c->N / tile, (float *)c->rowmaxB.p, c->stream));
+        }
         if (c->timing) HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
-        HIPCHK(c, launch_normmap_a(dX, in16, rows, cols, tile, c->packedA.p, (float *)c->nA.p, c->stream));
+        HIPCHK(c, launch_normmap_a(dX, in16, rows, cols, tile, c->packedA.p, (float *)c->nA.p,
+                                   prune ? (const float *)c->rowmaxB.p : nullptr, prune ? *prune_tau : 0.0f, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[2], c->stream)); c->ev_a = true; }
         c->have_a = true;
+        c->a_pruned = prune;
+        c->a_pruned_tau = prune ? *prune_tau : 0.0f;
     } else {
         if (c->have_a && c->K != rows) c->have_a = false;
+        if (c->a_pruned) c->have_a = false;     // pruned against the previous B's norms
         c->K = rows;
         c->N = cols;
         if ((rc = ensure(c, c->packedB, (size_t)rows * cols * 2))) return rc;
@@ -300,6 +315,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
 int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (!c || !dC) return SPAMM_EINVAL;
     if (!c->have_a || !c->have_b || !c->have_gate) return SPAMM_ESTATE;
+    if (c->a_pruned && !(c->tau >= c->a_pruned_tau)) return SPAMM_ESTATE;   // A's copy lacks tiles this tau keeps
     int rc = set_device(c);
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
@@ -324,6 +340,8 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     // same order as the reference: B's norm map first, then A's (cuSpAMM.cu:478-503)
     // an operand flagged for reuse must be resident with the same shape and tile
     if (reuse_a && !(c->have_a && c->tile == p->tile && c->M == p->M && c->K == p->K)) return SPAMM_ESTATE;
+    // a copy of A written by a tau-aware pass serves the same B and thresholds not below that tau only
+    if (reuse_a && c->a_pruned && !(reuse_b && p->tau >= c->a_pruned_tau)) return SPAMM_ESTATE;
     if (reuse_b && !(c->have_b && c->tile == p->tile && c->K == p->K && c->N == p->N)) return SPAMM_ESTATE;
     const bool a_eq_b = (p->flags & SPAMM_FLAG_A_EQ_B) != 0;
     if (a_eq_b) {
@@ -350,6 +368,7 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
             c->ev_a = c->ev_b = true;
         }
         c->have_a = c->have_b = true;
+        c->a_pruned = false;
         c->have_gate = false;
     } else if (!reuse_b) {
         if ((rc = normmap_any(c, SPAMM_ROLE_B, dB, in16, p->K, p->N, p->tile))) return rc;
@@ -361,7 +380,8 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     if (a_eq_b) {
         // done above
     } else if (!reuse_a) {
-        if ((rc = normmap_any(c, SPAMM_ROLE_A, dA, in16, p->M, p->K, p->tile))) return rc;
+        const bool prune = (p->flags & SPAMM_FLAG_PRUNE_A) != 0;
+        if ((rc = normmap_any(c, SPAMM_ROLE_A, dA, in16, p->M, p->K, p->tile, prune ? &p->tau : nullptr))) return rc;
     } else if (c->timing) {
         HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
         c->ev_a = true;
@@ -381,7 +401,7 @@ int spamm_multiply_f16(spamm_ctx *c, const spamm_params *p, const void *dAh, con
 
 int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_t row1, double *out3) {
     if (!c || !dC || !out3) return SPAMM_EINVAL;
-    if (!c->have_a || !c->have_b) return SPAMM_ESTATE;
+    if (!c->have_a || !c->have_b || c->a_pruned) return SPAMM_ESTATE;   // needs A's complete fp16 copy
     if (row0 < 0 || row1 > c->M || row0 >= row1 || row0 % 64 || row1 % 64 || c->N % 64 || c->K % 16)
         return SPAMM_EINVAL;
     int rc = set_device(c);
@@ -676,7 +696,7 @@ int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
     int64_t rows, cols;
     const void *packed;
     if (role == SPAMM_ROLE_A) {
-        if (!c->have_a) return SPAMM_ESTATE;
+        if (!c->have_a || c->a_pruned) return SPAMM_ESTATE;
         rows = c->M; cols = c->K; packed = c->packedA.p;
     } else if (role == SPAMM_ROLE_B) {
         if (!c->have_b) return SPAMM_ESTATE;
