@@ -75,7 +75,8 @@ def test_command_line_driver_is_built_and_checks_its_arguments():
     main = os.path.join(ROOT, "cuspamm_amd", "spamm_main")
     assert os.path.exists(main), "build it with `python -m cuspamm_amd.build`"
     for args, msg in ((["--tile", "48"], "tile must be"), (["--nonsense"], "unknown option"),
-                      (["--testtime", "3", "--warmup", "5"], "bad sizes")):
+                      (["--testtime", "3", "--warmup", "5"], "bad sizes"),
+                      (["--check", "--prune-a"], "complete fp16 copy")):
         proc = subprocess.run([main] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
         assert proc.returncode == 2 and msg in proc.stdout, proc.stdout
 
