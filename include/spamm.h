@@ -117,8 +117,9 @@ SPAMM_API int spamm_normmap_f16(spamm_ctx *ctx, int role, const void *dXh, int64
                                 int32_t tile);
 
 /* Stage 2 -- replaces the gating prologue of get_C_FP16_B32
- * (cuSpAMM.cu:302-334): per output tile the kept-k bitmap, the ascending
- * compacted k list and the count.  Uses the norm maps left by stage 1 (or by
+ * (cuSpAMM.cu:302-334): per output tile the kept-k bitmap and the count (the
+ * ascending compacted k list of :315-325 is the bitmap's set bits in order;
+ * spamm_get_klist materialises it).  Uses the norm maps left by stage 1 (or by
  * spamm_set_normmaps). */
 SPAMM_API int spamm_gate(spamm_ctx *ctx, float tau);
 
@@ -153,7 +154,8 @@ SPAMM_API int spamm_set_normmaps(spamm_ctx *ctx, const float *nA, const float *n
 /* Read-back helpers (host destination buffers; each synchronises the stream).
  *   normmap: row-major, role A [M/b x K/b], role B [K/b x N/b] (cuSpAMM.cu:438-439)
  *   counts:  int32 [nbM*nbN]
- *   klist:   uint16 [nbM*nbN*nbK], first counts[t] entries of each row valid
+ *   klist:   uint16 [nbM*nbN*nbK], first counts[t] entries of each row valid (built from the
+ *            mask by this call; the rest of each row is unspecified)
  *   mask:    uint64 [nbM*nbN*ceil(nbK/64)], bit k of tile t
  *   fp16:    the fp16 copy of an operand un-packed to row-major bit patterns */
 SPAMM_API int spamm_get_normmap(spamm_ctx *ctx, int role, float *host_out);

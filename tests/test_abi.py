@@ -38,6 +38,15 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(sp.SpammStats) == 40
 
 
+def test_flag_values_match_header():
+    from cuspamm_amd import api
+    text = open(os.path.join(ROOT, "include", "spamm.h")).read()
+    flags = dict(re.findall(r"#define\s+SPAMM_(FLAG_[A-Z_]+)\s+(\d+)u", text))
+    assert set(flags) == {"FLAG_A_EQ_B", "FLAG_TIMING", "FLAG_REUSE_A", "FLAG_REUSE_B", "FLAG_PRUNE_A"}
+    for name, value in flags.items():
+        assert getattr(api, name) == int(value), name
+
+
 def test_error_strings():
     import cuspamm_amd as sp
     L = sp.load_library()
