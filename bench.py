@@ -110,8 +110,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-literal", action="store_true", help="skip the one-off run of the literal lam=0.1 config")
     ap.add_argument("--skip-dense", action="store_true", help="skip the dense fp16 GEMM comparison")
-    ap.add_argument("--no-prune-a", action="store_true",
-                    help="timed multiplies without SPAMM_FLAG_PRUNE_A (the A pass then writes every fp16 tile)")
+    ap.add_argument("--no-prune", action="store_true",
+                    help="timed multiplies without SPAMM_FLAG_PRUNE (the A pass then writes every fp16 tile)")
     ap.add_argument("--cpu-budget", type=float, default=12.0, help="seconds of host GEMM in the CPU sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE/WRITE_SIZE)")
@@ -157,14 +157,14 @@ def main():
     # the timed steps run the path as a caller would (no per-stage events between the kernels).
     # tau is an argument of the call, so the A pass (second, as in the reference) can leave out
     # the fp16 copy of tiles that no product keeps: same C, mask and counts, fewer bytes written.
-    prune = not args.no_prune_a
+    prune = not args.no_prune
     for _ in range(args.warmup):
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune_a=prune)
+        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)
     torch.cuda.synchronize()
     stage = np.zeros(5)
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune_a=prune)
+        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / args.steps
@@ -172,21 +172,25 @@ def main():
     # re-run the same steps reading the events after each one (reading needs a sync, so it is
     # kept out of the wall-clock loop above)
     for _ in range(args.steps):
-        ctx.multiply(dA, dB, tile, tau, C=dC, timing=True, prune_a=prune)
+        ctx.multiply(dA, dB, tile, tau, C=dC, timing=True, prune=prune)
         st = ctx.get_stats()
         stage += [st.ms_normmap_b, st.ms_normmap_a, st.ms_gate, st.ms_gemm, st.ms_total]
     stage /= args.steps
     # bytes the A pass writes: tile (i, k) is copied iff fl32(nA[i,k] * max_j nB[k,j]) >= tau
     nA_h, nB_h = ctx.get_normmap(sp.ROLE_A), ctx.get_normmap(sp.ROLE_B)
+    # and the B pass every tile of non-zero norm
     a_tiles = nb * nb
-    a_written = int(np.count_nonzero(nA_h * nB_h.max(axis=1)[None, :] >= np.float32(tau))) if prune else a_tiles
+    pruned = prune and tau > 0
+    a_written = int(np.count_nonzero(nA_h * nB_h.max(axis=1)[None, :] >= np.float32(tau))) if pruned else a_tiles
+    b_written = int(np.count_nonzero(nB_h)) if pruned else a_tiles
     kept, total = int(st.kept_products), int(st.total_products)
     flops = kept * 2.0 * tile ** 3
     value = flops / (ms_step * 1e-3) / 1e12
     gemm_tflops = flops / (stage[3] * 1e-3) / 1e12
     nm_bytes = 4.0 * N * N + 2.0 * N * N + 4.0 * nb * nb               # per matrix, every tile written
     nm_bytes_a = 4.0 * N * N + 2.0 * tile * tile * a_written + 4.0 * nb * nb
-    nm_gbs = nm_bytes / (stage[0] * 1e-3) / 1e9                        # the B pass (always complete)
+    nm_bytes_b = 4.0 * N * N + 2.0 * tile * tile * b_written + 8.0 * nb * nb
+    nm_gbs = nm_bytes_b / (stage[0] * 1e-3) / 1e9                      # the B pass
 
     out = {
         "metric": "spamm_effective_tflops_kept_tiles",
@@ -207,7 +211,7 @@ def main():
             "name": args.workload, "N": N, "tile": tile, "tau": tau,
             "kept_products": kept, "total_products": total,
             "kept_fraction": round(kept / total, 5),
-            "prune_a": prune,
+            "prune": prune,
         },
         "stage_ms": {"normmap_b": round(stage[0], 4), "normmap_a": round(stage[1], 4), "gate": round(stage[2], 4),
                      "gemm": round(stage[3], 4), "sum_events": round(stage[4], 4)},
@@ -225,12 +229,13 @@ def main():
             "kernel": "k_normmap<%d, B role> (fp32->fp16 + tile norms)" % tile, "bound": "hbm",
             "achieved": round(nm_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": round(nm_gbs / PEAK_HBM_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("normmap"),
-            "bytes_per_launch": nm_bytes, "avg_launch_ms": round(stage[0], 4),
+            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("normmap_b_pruned" if pruned else "normmap"),
+            "bytes_per_launch": nm_bytes_b, "avg_launch_ms": round(stage[0], 4),
+            "tiles_written": b_written, "tiles": a_tiles, "bytes_per_launch_all_tiles": nm_bytes,
             "a_pass": {"tiles_written": a_written, "tiles": a_tiles, "bytes_per_launch": nm_bytes_a,
                        "avg_launch_ms": round(stage[1], 4),
                        "achieved": round(nm_bytes_a / (stage[1] * 1e-3) / 1e9, 1),
-                       "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("normmap_a_pruned") if prune
+                       "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("normmap_a_pruned") if pruned
                        else MEASURED_TRAFFIC.get(args.workload, {}).get("normmap")},
         },
     }
@@ -305,7 +310,7 @@ def main():
         same_c = None
         if prune:
             plain = ctx.multiply(dA, dB, tile, tau).clone()
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune_a=prune)      # the call that was timed
+        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)      # the call that was timed
         if prune:
             same_c = bool(torch.equal(plain, dC))
             del plain
@@ -334,7 +339,7 @@ def main():
             "fp64_dense_frobenius": float("%.4e" % np.sqrt(d_nrm)),
             "tau_bound_frobenius": float("%.4e" % np.sqrt(bound)),
             "rows_checked": len(rows), "rows_vs_fp64": 2,
-            "prune_a_c_bit_identical_to_plain_call": same_c,
+            "prune_c_bit_identical_to_plain_call": same_c,
         }
     elif not args.no_cpu_baseline:
         out["cpu_baseline"] = None

@@ -17,7 +17,7 @@ FLAG_A_EQ_B = 1
 FLAG_TIMING = 2
 FLAG_REUSE_A = 4
 FLAG_REUSE_B = 8
-FLAG_PRUNE_A = 16
+FLAG_PRUNE = 16
 
 OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV = 0, -1, -2, -3, -4, -5
 
@@ -168,11 +168,11 @@ class SpammContext:
 
     # -- the multiply call
     def multiply(self, A, B, tile, tau, C=None, timing=False, reuse_a=False, reuse_b=False, a_eq_b=False,
-                 prune_a=False):
+                 prune=False):
         """C = SpAMM(A, B).  fp32 or fp16 inputs (both the same dtype).  With reuse_a / reuse_b the
         operand's fp16 copy and norm map from the previous call are kept (pass the same tensor, it
-        only supplies the shape).  prune_a: tau-aware A pass (same C, mask and counts; A's fp16 copy
-        is then incomplete, see SPAMM_FLAG_PRUNE_A)."""
+        only supplies the shape).  prune: tau-aware conversion passes (same C, mask and counts; the
+        fp16 copies are then incomplete, see SPAMM_FLAG_PRUNE)."""
         import torch
         if A.dim() != 2 or B.dim() != 2:
             raise ValueError("A and B must be matrices")
@@ -186,7 +186,7 @@ class SpammContext:
             C = torch.empty((M, N), dtype=torch.float32, device=A.device)
         flags = ((FLAG_TIMING if timing else 0) | (FLAG_REUSE_A if reuse_a else 0) |
                  (FLAG_REUSE_B if reuse_b else 0) | (FLAG_A_EQ_B if a_eq_b else 0) |
-                 (FLAG_PRUNE_A if prune_a else 0))
+                 (FLAG_PRUNE if prune else 0))
         p = SpammParams(M, K, N, int(tile), float(tau), flags, 0)
         if A.dtype == torch.float16:
             _check(self._lib.spamm_multiply_f16(self._h, ctypes.byref(p), _devptr(A, "float16"),

@@ -178,15 +178,17 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             }
         }
     };
-    // norms: one wave per tile, canonical order.  With `prune` (A role, tau known, B's norm map
-    // done) the wave also decides whether any product can keep the tile: fl(nA[i,k] * nB[k,j]) <=
-    // fl(nA[i,k] * max_j nB[k,j]) because rounding is monotone, so a tile whose product with the
-    // row maximum is below tau is never read by the GEMM and its fp16 copy need not be written.
+    // norms: one wave per tile, canonical order.  With `prune` (tau known and positive) the wave
+    // also decides whether any product can keep the tile: fl(n * n') <= fl(n * bound) for every
+    // partner norm n' <= bound because rounding is monotone, so a tile whose product with the
+    // bound is below tau is never read by the GEMM and its fp16 copy need not be written.  The
+    // bound is max_j nB[k,j] for the A pass (B's norm map is complete by then) and the largest
+    // finite float for the B pass, which runs first: there only tiles of norm zero are left out.
     auto norms = [&](bool as_b, float *__restrict__ nmo, float *__restrict__ nmTo, bool prune) {
         for (int tt = wave; tt < TPS; tt += 4) {
             const int64_t Jt = sc * TPS + tt;
             if (Jt >= nbc) break;
-            const float rmax = prune ? rowmax[Jt] : 0.0f;
+            const float rmax = prune ? (rowmax != nullptr ? rowmax[Jt] : 3.402823466e+38f) : 0.0f;
             float partial = 0.0f;
 #pragma unroll
             for (int it = 0; it < STEPS; it++) {
@@ -209,7 +211,7 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
     if (ROLE == 0) {
         stage_a();
         __syncthreads();
-        if (rowmax != nullptr) {
+        if (tau_skip > 0.0f) {
             norms(false, nm, nullptr, true);
             __syncthreads();
             copy_out(false, packed, true);
@@ -219,7 +221,13 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
     } else if (ROLE == 1) {
         stage_b();
         __syncthreads();
-        emit(true, packed, nm, nmT);
+        if (tau_skip > 0.0f) {
+            norms(true, nm, nmT, true);
+            __syncthreads();
+            copy_out(true, packed, true);
+        } else {
+            emit(true, packed, nm, nmT);
+        }
     } else {
         stage_a();
         __syncthreads();
@@ -349,9 +357,9 @@ hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void
 }
 
 hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
-                            float *nm, float *nmT, hipStream_t s) {
-    return in16 ? launch_normmap<1, true>(X, rows, cols, tile, packed, nm, nmT, s)
-                : launch_normmap<1, false>(X, rows, cols, tile, packed, nm, nmT, s);
+                            float *nm, float *nmT, float tau_skip, hipStream_t s) {
+    return in16 ? launch_normmap<1, true>(X, rows, cols, tile, packed, nm, nmT, s, nullptr, nullptr, nullptr, tau_skip)
+                : launch_normmap<1, false>(X, rows, cols, tile, packed, nm, nmT, s, nullptr, nullptr, nullptr, tau_skip);
 }
 
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,

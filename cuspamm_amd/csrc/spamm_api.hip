@@ -38,6 +38,8 @@ struct spamm_ctx {
     // a_pruned_tau are missing, so the copy serves a GEMM only for tau >= a_pruned_tau
     bool a_pruned = false;
     float a_pruned_tau = 0.0f;
+    // B's fp16 copy lacks its tiles of norm zero: it serves any tau > 0
+    bool b_pruned = false;
 
     DevBuf packedA, packedB, nA, nB, nBt, rowmaxB;
     DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, sched, kept_total;
@@ -118,7 +120,7 @@ void reset_shape(spamm_ctx *c, int tile) {
     c->tile = tile;
     c->M = c->K = c->N = 0;
     c->have_a = c->have_b = c->have_gate = false;
-    c->a_pruned = false;
+    c->a_pruned = c->b_pruned = false;
 }
 
 int copy_out(spamm_ctx *c, const void *dev, void *host, size_t bytes) {
@@ -223,7 +225,7 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
         if ((rc = ensure(c, c->packedA, (size_t)rows * cols * 2))) return rc;
         if ((rc = ensure(c, c->nA, nt * 4))) return rc;
         // tau-aware pass: needs B's norm map of the same K (the caller checked have_b)
-        const bool prune = prune_tau != nullptr && c->have_b && c->nB.p;
+        const bool prune = prune_tau != nullptr && *prune_tau > 0.0f && c->have_b && c->nB.p;
         if (prune) {
             if ((rc = ensure(c, c->rowmaxB, (size_t)(cols / tile) * 4))) return rc;
             HIPCHK(c, launch_rowmax((const float *)c->nB.p, cols / tile, c->N / tile, (float *)c->rowmaxB.p, c->stream));
@@ -244,10 +246,12 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
         if ((rc = ensure(c, c->nB, nt * 4))) return rc;
         if ((rc = ensure(c, c->nBt, nt * 4))) return rc;
         if (c->timing) HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
+        const bool prune = prune_tau != nullptr && *prune_tau > 0.0f;
         HIPCHK(c, launch_normmap_b(dX, in16, rows, cols, tile, c->packedB.p, (float *)c->nB.p,
-                                   (float *)c->nBt.p, c->stream));
+                                   (float *)c->nBt.p, prune ? *prune_tau : 0.0f, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[1], c->stream)); c->ev_b = true; }
         c->have_b = true;
+        c->b_pruned = prune;
     }
     c->have_gate = false;
     return SPAMM_OK;
@@ -316,6 +320,7 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (!c || !dC) return SPAMM_EINVAL;
     if (!c->have_a || !c->have_b || !c->have_gate) return SPAMM_ESTATE;
     if (c->a_pruned && !(c->tau >= c->a_pruned_tau)) return SPAMM_ESTATE;   // A's copy lacks tiles this tau keeps
+    if (c->b_pruned && !(c->tau > 0.0f)) return SPAMM_ESTATE;               // B's copy lacks its zero tiles
     int rc = set_device(c);
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
@@ -342,6 +347,7 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     if (reuse_a && !(c->have_a && c->tile == p->tile && c->M == p->M && c->K == p->K)) return SPAMM_ESTATE;
     // a copy of A written by a tau-aware pass serves the same B and thresholds not below that tau only
     if (reuse_a && c->a_pruned && !(reuse_b && p->tau >= c->a_pruned_tau)) return SPAMM_ESTATE;
+    if (reuse_b && c->b_pruned && !(p->tau > 0.0f)) return SPAMM_ESTATE;
     if (reuse_b && !(c->have_b && c->tile == p->tile && c->K == p->K && c->N == p->N)) return SPAMM_ESTATE;
     const bool a_eq_b = (p->flags & SPAMM_FLAG_A_EQ_B) != 0;
     if (a_eq_b) {
@@ -368,10 +374,11 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
             c->ev_a = c->ev_b = true;
         }
         c->have_a = c->have_b = true;
-        c->a_pruned = false;
+        c->a_pruned = c->b_pruned = false;
         c->have_gate = false;
     } else if (!reuse_b) {
-        if ((rc = normmap_any(c, SPAMM_ROLE_B, dB, in16, p->K, p->N, p->tile))) return rc;
+        const bool prune = (p->flags & SPAMM_FLAG_PRUNE) != 0;
+        if ((rc = normmap_any(c, SPAMM_ROLE_B, dB, in16, p->K, p->N, p->tile, prune ? &p->tau : nullptr))) return rc;
     } else if (c->timing) {
         HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
         HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
@@ -380,7 +387,7 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     if (a_eq_b) {
         // done above
     } else if (!reuse_a) {
-        const bool prune = (p->flags & SPAMM_FLAG_PRUNE_A) != 0;
+        const bool prune = (p->flags & SPAMM_FLAG_PRUNE) != 0;
         if ((rc = normmap_any(c, SPAMM_ROLE_A, dA, in16, p->M, p->K, p->tile, prune ? &p->tau : nullptr))) return rc;
     } else if (c->timing) {
         HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
@@ -401,7 +408,7 @@ int spamm_multiply_f16(spamm_ctx *c, const spamm_params *p, const void *dAh, con
 
 int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_t row1, double *out3) {
     if (!c || !dC || !out3) return SPAMM_EINVAL;
-    if (!c->have_a || !c->have_b || c->a_pruned) return SPAMM_ESTATE;   // needs A's complete fp16 copy
+    if (!c->have_a || !c->have_b || c->a_pruned || c->b_pruned) return SPAMM_ESTATE;   // needs complete fp16 copies
     if (row0 < 0 || row1 > c->M || row0 >= row1 || row0 % 64 || row1 % 64 || c->N % 64 || c->K % 16)
         return SPAMM_EINVAL;
     int rc = set_device(c);
@@ -699,7 +706,7 @@ int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
         if (!c->have_a || c->a_pruned) return SPAMM_ESTATE;
         rows = c->M; cols = c->K; packed = c->packedA.p;
     } else if (role == SPAMM_ROLE_B) {
-        if (!c->have_b) return SPAMM_ESTATE;
+        if (!c->have_b || c->b_pruned) return SPAMM_ESTATE;
         rows = c->K; cols = c->N; packed = c->packedB.p;
     } else {
         return SPAMM_EINVAL;

@@ -63,13 +63,14 @@ struct GateBuffers {
     int64_t *kept_total;    // [1]  kept products
 };
 
-// rowmax != nullptr: tau-aware pass, the fp16 copy of tile (i, k) is written only if
+// tau_skip > 0: tau-aware pass, the fp16 copy of tile (i, k) is written only if
 // fl(nA[i,k] * rowmax[k]) >= tau_skip (rowmax[k] = max_j nB[k,j], launch_rowmax)
 hipError_t launch_normmap_a(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
                             float *nm, const float *rowmax, float tau_skip, hipStream_t s);
 hipError_t launch_rowmax(const float *nB, int64_t nbK, int64_t nbN, float *rowmax, hipStream_t s);
+// tau_skip > 0: the fp16 copy of tiles of norm zero is not written (no product with them reaches tau)
 hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,
-                            float *nm, float *nmT, hipStream_t s);
+                            float *nm, float *nmT, float tau_skip, hipStream_t s);
 // A = B (square): one pass over X for both operand roles
 hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void *packedA, float *nmA,
                              void *packedB, float *nmB, float *nmBt, hipStream_t s);

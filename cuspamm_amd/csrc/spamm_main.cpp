@@ -10,7 +10,7 @@
 //
 //   spamm_main [--M m] [--K k] [--N n] [--tile 32|64|128] [--tau t | --ratio r | --tune r]
 //              [--gen exp|alg|ones] [--c c] [--v v] [--a-csv f --b-csv f | --a-mtx f --b-mtx f]
-//              [--testtime n] [--warmup n] [--check | --prune-a] [--device d]
+//              [--testtime n] [--warmup n] [--check | --prune] [--device d]
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -37,7 +37,7 @@ int main(int argc, char **argv) {
     bool cv_given = false;
     std::string a_csv, b_csv, a_mtx, b_mtx;
     int testtime = 10, warmup = 5, device = 0;         // TESTTIME, WARMUP, para.h:4-5
-    bool check = false, prune_a = false;
+    bool check = false, prune = false;
     for (int i = 1; i < argc; i++) {
         const std::string o = argv[i];
         auto val = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };
@@ -59,12 +59,12 @@ int main(int argc, char **argv) {
         else if (o == "--warmup") warmup = atoi(val());
         else if (o == "--device") device = atoi(val());
         else if (o == "--check") check = true;
-        else if (o == "--prune-a") prune_a = true;
+        else if (o == "--prune") prune = true;
         else { fprintf(stderr, "spamm_main: unknown option %s\n", o.c_str()); return 2; }
     }
     if (gen == "exp" && !cv_given) { c = 1.0f; v = 0.1f; }    // getDecayMatrixExp(h, 1, 0.1, ...), cuSpAMM.cu:426-427
     if (tile != 32 && tile != 64 && tile != 128) { fprintf(stderr, "spamm_main: tile must be 32, 64 or 128\n"); return 2; }
-    if (check && prune_a) { fprintf(stderr, "spamm_main: --check needs A's complete fp16 copy, --prune-a leaves tiles out\n"); return 2; }
+    if (check && prune) { fprintf(stderr, "spamm_main: --check needs A's complete fp16 copy, --prune leaves tiles out\n"); return 2; }
     if (inM <= 0 || inK <= 0 || inN <= 0 || testtime <= warmup + 1) { fprintf(stderr, "spamm_main: bad sizes\n"); return 2; }
     // padded dimensions (main.h:54-56)
     const long long M = (inM + tile - 1) / tile * tile, K = (inK + tile - 1) / tile * tile, N = (inN + tile - 1) / tile * tile;
@@ -109,7 +109,7 @@ int main(int argc, char **argv) {
 
     spamm_params p;
     memset(&p, 0, sizeof(p));
-    p.M = M; p.K = K; p.N = N; p.tile = tile; p.tau = (float)norm_init; p.flags = SPAMM_FLAG_TIMING | (prune_a ? SPAMM_FLAG_PRUNE_A : 0u);
+    p.M = M; p.K = K; p.N = N; p.tile = tile; p.tau = (float)norm_init; p.flags = SPAMM_FLAG_TIMING | (prune ? SPAMM_FLAG_PRUNE : 0u);
     if (ratio >= 0.0 || tune >= 0.0) {
         // valid-ratio driven tau: exact order statistic, or the reference's bisection (main.h:35-38)
         if ((rc = spamm_normmap_f32(ctx, SPAMM_ROLE_B, dB, K, N, tile))) return fail("norm map of B", rc);

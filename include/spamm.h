@@ -45,15 +45,18 @@ extern "C" {
 #define SPAMM_FLAG_TIMING 2u     /* record per-stage HIP events (spamm_get_stats) */
 #define SPAMM_FLAG_REUSE_A 4u    /* A's fp16 copy and norm map from an earlier call are reused (dA ignored) */
 #define SPAMM_FLAG_REUSE_B 8u    /* same for B: e.g. one B against many A, or matrix powers */
-#define SPAMM_FLAG_PRUNE_A 16u   /* tau-aware A pass: the fp16 copy of tile A_ik is written only if some product can
-                                  * keep it, fl(|A_ik| * max_j |B_kj|) >= tau (exact: fp32 rounding is monotone, so
-                                  * every product of a skipped tile fails the gate).  C, mask and counts are
-                                  * identical to a call without the flag; the pass writes less.  Afterwards A's
-                                  * copy is incomplete: SPAMM_FLAG_REUSE_A is accepted only together with
-                                  * SPAMM_FLAG_REUSE_B and tau' >= tau, and spamm_get_fp16(A) and
-                                  * spamm_error_vs_dense_f64 return SPAMM_ESTATE until A is converted again
-                                  * without the flag.  Ignored with SPAMM_FLAG_A_EQ_B.  No counterpart in the
-                                  * reference, which converts on the host outside its timed region (tool.cu:418,432). */
+#define SPAMM_FLAG_PRUNE 16u     /* tau-aware conversion passes (tau > 0): the fp16 copy of a tile is written only if some
+                                  * product can keep it.  A tile A_ik: fl(|A_ik| * max_j |B_kj|) >= tau (B's norms are
+                                  * complete when A's pass runs).  B tile B_kj: |B_kj| > 0 (B's pass runs first; a
+                                  * tile of norm zero fails the gate against any A).  Exact: fp32 rounding is
+                                  * monotone, so every product of a skipped tile fails the gate.  C, mask and counts
+                                  * are identical to a call without the flag; the passes write less.  Afterwards the
+                                  * copies are incomplete: SPAMM_FLAG_REUSE_A is accepted only together with
+                                  * SPAMM_FLAG_REUSE_B and tau' >= tau, SPAMM_FLAG_REUSE_B only with tau' > 0, and
+                                  * spamm_get_fp16 and spamm_error_vs_dense_f64 return SPAMM_ESTATE until the
+                                  * operand is converted again without the flag.  Ignored with SPAMM_FLAG_A_EQ_B and
+                                  * for tau <= 0.  No counterpart in the reference, which converts on the host
+                                  * outside its timed region (tool.cu:418,432). */
 
 /* Run-time form of the reference's compile-time configuration:
  * M,K,N <- inM,inK,inN (para.h:6-8) already padded to a tile multiple

@@ -42,7 +42,7 @@ def test_flag_values_match_header():
     from cuspamm_amd import api
     text = open(os.path.join(ROOT, "include", "spamm.h")).read()
     flags = dict(re.findall(r"#define\s+SPAMM_(FLAG_[A-Z_]+)\s+(\d+)u", text))
-    assert set(flags) == {"FLAG_A_EQ_B", "FLAG_TIMING", "FLAG_REUSE_A", "FLAG_REUSE_B", "FLAG_PRUNE_A"}
+    assert set(flags) == {"FLAG_A_EQ_B", "FLAG_TIMING", "FLAG_REUSE_A", "FLAG_REUSE_B", "FLAG_PRUNE"}
     for name, value in flags.items():
         assert getattr(api, name) == int(value), name
 
@@ -85,7 +85,7 @@ def test_command_line_driver_is_built_and_checks_its_arguments():
     assert os.path.exists(main), "build it with `python -m cuspamm_amd.build`"
     for args, msg in ((["--tile", "48"], "tile must be"), (["--nonsense"], "unknown option"),
                       (["--testtime", "3", "--warmup", "5"], "bad sizes"),
-                      (["--check", "--prune-a"], "complete fp16 copy")):
+                      (["--check", "--prune"], "complete fp16 copy")):
         proc = subprocess.run([main] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
         assert proc.returncode == 2 and msg in proc.stdout, proc.stdout
 

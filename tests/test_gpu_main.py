@@ -47,7 +47,7 @@ def test_reference_generators_through_the_driver(orc, gen, c, v, tile, tau):
 def test_driver_pads_and_tunes(orc):
     # dimensions that are not tile multiples are padded up (main.h:54-56); --ratio picks tau on the device
     out = _run(["--M", 1000, "--K", 900, "--N", 1100, "--tile", 64, "--gen", "exp", "--c", 1.0, "--v", 0.99,
-                "--ratio", 0.3, "--testtime", 3, "--warmup", 0, "--prune-a"])
+                "--ratio", 0.3, "--testtime", 3, "--warmup", 0, "--prune"])
     assert "input parameters: M=1024 K=960 N=1152" in out
     ach = float(re.search(r"valid ratio=([0-9.]+)", out).group(1))
     kept, total = map(int, re.search(r"valid products=(\d+) of (\d+)", out).groups())

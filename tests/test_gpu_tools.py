@@ -101,45 +101,54 @@ def test_a_equals_b_single_pass(orc, ctx, tile):
 
 
 @pytest.mark.parametrize("tile", [32, 64, 128])
-def test_tau_aware_a_pass_gives_the_same_product(orc, ctx, tile):
-    """SPAMM_FLAG_PRUNE_A: A tiles that no product can keep are not copied; C, mask, counts and norm
-    maps must not change.  The workspace is first filled with a loud A so that a GEMM reading a
-    skipped tile would show."""
+def test_tau_aware_passes_give_the_same_product(orc, ctx, tile):
+    """SPAMM_FLAG_PRUNE: A tiles that no product can keep and B tiles of norm zero are not copied;
+    C, mask, counts and norm maps must not change.  The workspace is first filled with loud
+    operands so that a GEMM reading a skipped tile would show."""
     import torch
     import cuspamm_amd as sp
     M, K, N = 4 * 256, 3 * 256, 2 * 256 + tile
-    tab = orc.decay_table("exp", max(M, K, N), 0.02)
+    tab = orc.decay_table("exp", max(M, K, N), 0.05)      # exactly zero in fp16 beyond |i - j| ~ 333
     A = _dev(orc.fill_decay(M, K, tab, 1))
     B = _dev(orc.fill_decay(K, N, tab, 2))
     ctx.normmap_f32(1, B, tile)
     ctx.normmap_f32(0, A, tile)
-    tau, ach = ctx.tau_for_ratio(0.15)
-    assert 0.05 < ach < 0.3
+    tau, ach = ctx.tau_for_ratio(0.05)
+    assert tau > 0 and 0.01 < ach < 0.2
     Cref = ctx.multiply(A, B, tile, tau).clone()
-    mask, counts, nA = ctx.get_mask(), ctx.get_counts(), ctx.get_normmap(0)
+    mask, counts, nA, nB = ctx.get_mask(), ctx.get_counts(), ctx.get_normmap(0), ctx.get_normmap(1)
     kept = ctx.get_stats().kept_products
-    # the checker's kept set says which A tiles are needed at all: some must be skippable here
+    # the checker's kept set says which A tiles are needed at all: some must be skippable here,
+    # and some B tiles must be exactly zero
     needed = np.unpackbits(mask.view(np.uint8), axis=-1, bitorder="little")[..., :K // tile].any(axis=1)
     assert 0 < needed.sum() < needed.size
-    ctx.multiply(torch.full_like(A, 1000.0), B, tile, 0.0)      # every tile of the workspace copy is now loud
-    C = ctx.multiply(A, B, tile, tau, prune_a=True)
+    assert 0 < np.count_nonzero(nB == 0) < nB.size
+    loud = ctx.multiply(torch.full_like(A, 1000.0), torch.full_like(B, 1000.0), tile, 0.0)   # both workspace copies are now loud
+    assert float(loud.min()) > 0
+    C = ctx.multiply(A, B, tile, tau, prune=True)
     assert torch.equal(C, Cref)
     assert np.array_equal(ctx.get_mask(), mask) and np.array_equal(ctx.get_counts(), counts)
     assert np.array_equal(ctx.get_normmap(0).view(np.uint32), nA.view(np.uint32))
+    assert np.array_equal(ctx.get_normmap(1).view(np.uint32), nB.view(np.uint32))
     assert ctx.get_stats().kept_products == kept
-    # the incomplete copy is fenced off
-    for call in (lambda: ctx.get_fp16(0), lambda: ctx.error_vs_dense(C),
+    # the incomplete copies are fenced off
+    for call in (lambda: ctx.get_fp16(0), lambda: ctx.get_fp16(1), lambda: ctx.error_vs_dense(C),
                  lambda: ctx.multiply(A, B, tile, tau * 0.5, reuse_a=True, reuse_b=True),
-                 lambda: ctx.multiply(A, B, tile, tau, reuse_a=True)):
+                 lambda: ctx.multiply(A, B, tile, tau, reuse_a=True),
+                 lambda: ctx.multiply(A, B, tile, 0.0, reuse_b=True)):
         with pytest.raises(sp.SpammError) as ei:
             call()
         assert ei.value.code == -4
-    # ... but serves the same B at the same or a larger threshold
-    ctx.multiply(A, B, tile, tau, prune_a=True)
+    # ... but serve the same operands at the same or a larger threshold
+    ctx.multiply(A, B, tile, tau, prune=True)
     C2 = ctx.multiply(A, B, tile, tau * 2, reuse_a=True, reuse_b=True).clone()
+    C3 = ctx.multiply(A, B, tile, tau * 0.5, reuse_b=True).clone()        # B's copy serves any tau > 0
     assert torch.equal(C2, ctx.multiply(A, B, tile, tau * 2))
-    # and a plain call makes it whole again
+    assert torch.equal(C3, ctx.multiply(A, B, tile, tau * 0.5))
+    # and a plain call makes them whole again
     assert np.array_equal(ctx.get_fp16(0), orc.f32_to_f16_bits(A.cpu().numpy()))
-    # tau = 0 and tau = inf through the flag
-    assert torch.equal(ctx.multiply(A, B, tile, 0.0, prune_a=True), ctx.multiply(A, B, tile, 0.0))
-    assert float(ctx.multiply(A, B, tile, float("inf"), prune_a=True).abs().max()) == 0.0
+    assert np.array_equal(ctx.get_fp16(1), orc.f32_to_f16_bits(B.cpu().numpy()))
+    # tau = 0 (nothing may be left out) and tau = inf through the flag
+    assert torch.equal(ctx.multiply(A, B, tile, 0.0, prune=True), ctx.multiply(A, B, tile, 0.0))
+    assert np.array_equal(ctx.get_fp16(1), orc.f32_to_f16_bits(B.cpu().numpy()))
+    assert float(ctx.multiply(A, B, tile, float("inf"), prune=True).abs().max()) == 0.0
