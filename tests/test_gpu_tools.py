@@ -30,6 +30,7 @@ def test_fp16_inputs_equal_fp32_inputs_of_the_same_values(orc, ctx, tile):
     assert np.array_equal(ctx.get_normmap(0).view(np.uint32), nA16.view(np.uint32))
     assert np.array_equal(ctx.get_normmap(1).view(np.uint32), nB16.view(np.uint32))
     assert torch.equal(C16, C32)
+    assert torch.equal(C16, ctx.multiply(A, B, tile, tau, prune=True))      # tau-aware passes on fp16 inputs
     kept = ctx.get_stats().kept_products
     assert 0 < kept < (M // tile) * (K // tile) * (N // tile)
 
