@@ -90,6 +90,18 @@ def test_command_line_driver_is_built_and_checks_its_arguments():
         assert proc.returncode == 2 and msg in proc.stdout, proc.stdout
 
 
+def test_missing_library_fails_loudly():
+    # no CPU or PyTorch fallback: without the built HIP library the package refuses to work
+    import subprocess
+    import sys
+    code = ("import cuspamm_amd as sp\n"
+            "try:\n    sp.load_library()\nexcept ImportError as e:\n    print('refused:', e)\n")
+    env = dict(os.environ, SPAMM_LIBRARY_PATH="/nonexistent/libspamm_gfx950.so")
+    proc = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0 and "refused:" in proc.stdout and "no CPU or PyTorch fallback" in proc.stdout, proc.stdout
+
+
 def test_product_package_never_imports_the_oracle():
     # the checker is test infrastructure: nothing under cuspamm_amd/ may reference it
     pkg = os.path.join(ROOT, "cuspamm_amd")
