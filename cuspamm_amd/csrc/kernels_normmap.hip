@@ -229,13 +229,27 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             emit(true, packed, nm, nmT);
         }
     } else {
+        // one pass for both roles: no row maxima yet, so only tiles of norm zero are left out
+        const bool prune = tau_skip > 0.0f;
         stage_a();
         __syncthreads();
-        emit(false, packed, nm, nullptr);
+        if (prune) {
+            norms(false, nm, nullptr, true);
+            __syncthreads();
+            copy_out(false, packed, true);
+        } else {
+            emit(false, packed, nm, nullptr);
+        }
         __syncthreads();
         stage_b();
         __syncthreads();
-        emit(true, packed2, nm2, nmT);
+        if (prune) {
+            norms(true, nm2, nmT, true);
+            __syncthreads();
+            copy_out(true, packed2, true);
+        } else {
+            emit(true, packed2, nm2, nmT);
+        }
     }
 }
 
@@ -351,9 +365,9 @@ hipError_t launch_rowmax(const float *nB, int64_t nbK, int64_t nbN, float *rowma
 }
 
 hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void *packedA, float *nmA,
-                             void *packedB, float *nmB, float *nmBt, hipStream_t s) {
-    return in16 ? launch_normmap<2, true>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB)
-                : launch_normmap<2, false>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB);
+                             void *packedB, float *nmB, float *nmBt, float tau_skip, hipStream_t s) {
+    return in16 ? launch_normmap<2, true>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB, nullptr, tau_skip)
+                : launch_normmap<2, false>(X, n, n, tile, packedA, nmA, nmBt, s, packedB, nmB, nullptr, tau_skip);
 }
 
 hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols, int tile, void *packed,

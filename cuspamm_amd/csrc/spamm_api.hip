@@ -366,15 +366,17 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
         if ((rc = ensure(c, c->nBt, nt * 4))) return rc;
         c->M = c->K = c->N = n;
         if (c->timing) HIPCHK(c, hipEventRecord(c->ev[0], c->stream));
+        const bool prune = (p->flags & SPAMM_FLAG_PRUNE) != 0 && p->tau > 0.0f;
         HIPCHK(c, launch_normmap_ab(dA, in16, n, p->tile, c->packedA.p, (float *)c->nA.p, c->packedB.p,
-                                    (float *)c->nB.p, (float *)c->nBt.p, c->stream));
+                                    (float *)c->nB.p, (float *)c->nBt.p, prune ? p->tau : 0.0f, c->stream));
         if (c->timing) {
             HIPCHK(c, hipEventRecord(c->ev[1], c->stream));
             HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
             c->ev_a = c->ev_b = true;
         }
         c->have_a = c->have_b = true;
-        c->a_pruned = c->b_pruned = false;
+        c->a_pruned = c->b_pruned = prune;       // both copies lack their tiles of norm zero:
+        c->a_pruned_tau = 1.0e-45f;              // they serve any tau > 0 (smallest positive float)
         c->have_gate = false;
     } else if (!reuse_b) {
         const bool prune = (p->flags & SPAMM_FLAG_PRUNE) != 0;

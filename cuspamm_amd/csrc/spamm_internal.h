@@ -73,7 +73,7 @@ hipError_t launch_normmap_b(const void *X, bool in16, int64_t rows, int64_t cols
                             float *nm, float *nmT, float tau_skip, hipStream_t s);
 // A = B (square): one pass over X for both operand roles
 hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void *packedA, float *nmA,
-                             void *packedB, float *nmB, float *nmBt, hipStream_t s);
+                             void *packedB, float *nmB, float *nmBt, float tau_skip, hipStream_t s);
 // error report tooling (kernels_tools.hip)
 hipError_t launch_error_vs_dense(const void *packedA, const void *packedB, int64_t M, int64_t K, int64_t N,
                                  int tile, const float *C, int64_t row0, int64_t row1, double *out3,

@@ -54,7 +54,8 @@ extern "C" {
                                   * copies are incomplete: SPAMM_FLAG_REUSE_A is accepted only together with
                                   * SPAMM_FLAG_REUSE_B and tau' >= tau, SPAMM_FLAG_REUSE_B only with tau' > 0, and
                                   * spamm_get_fp16 and spamm_error_vs_dense_f64 return SPAMM_ESTATE until the
-                                  * operand is converted again without the flag.  Ignored with SPAMM_FLAG_A_EQ_B and
+                                  * operand is converted again without the flag.  With SPAMM_FLAG_A_EQ_B (one pass, no
+                                  * row maxima yet) only tiles of norm zero are left out, in both copies.  Ignored
                                   * for tau <= 0.  No counterpart in the reference, which converts on the host
                                   * outside its timed region (tool.cu:418,432). */
 

@@ -85,7 +85,7 @@ def test_a_equals_b_single_pass(orc, ctx, tile):
     import torch
     import cuspamm_amd as sp
     n = 1024
-    tab = orc.decay_table("exp", n, 0.5 if tile == 32 else 0.02)
+    tab = orc.decay_table("exp", n, 0.5 if tile == 32 else 0.05)
     X = _dev(orc.fill_decay(n, n, tab, 1))
     tau = 1e-4 if tile == 32 else 2.0
     C2 = ctx.multiply(X, X, tile, tau).clone()
@@ -99,6 +99,17 @@ def test_a_equals_b_single_pass(orc, ctx, tile):
     assert 0 < kept < (n // tile) ** 3
     with pytest.raises(sp.SpammError):                       # the flag needs the same pointer and a square problem
         ctx.multiply(X, X.clone(), tile, tau, a_eq_b=True)
+    # the single pass with the tau-aware flag: tiles of norm zero are left out of both copies
+    # (exp(-0.5 d) is exactly zero in fp16 beyond d = 33, exp(-0.05 d) beyond d = 333)
+    assert np.count_nonzero(ref[1] == 0) > 0
+    ctx.multiply(torch.full_like(X, 1000.0), X, tile, 0.0)   # loud workspace
+    assert torch.equal(ctx.multiply(X, X, tile, tau, a_eq_b=True, prune=True), C2)
+    assert np.array_equal(ctx.get_mask(), ref[0])
+    with pytest.raises(sp.SpammError):
+        ctx.get_fp16(0)
+    with pytest.raises(sp.SpammError):
+        ctx.get_fp16(1)
+    assert torch.equal(ctx.multiply(X, X, tile, tau * 3, reuse_a=True, reuse_b=True), ctx.multiply(X, X, tile, tau * 3))
 
 
 @pytest.mark.parametrize("tile", [32, 64, 128])
