@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # They describe the committed kernels and are None for other workloads.
 MEASURED_TRAFFIC = {
     # fetch counter x 2.0 (a plain 1 GiB copy reads 524303 KiB on FETCH_SIZE), write counter x 1.0
-    "headline": {"gemm": 3.6819e9, "normmap": 1.6115e9, "normmap_a_pruned": 1.3145e9, "normmap_b_pruned": 1.3989e9},
+    "headline": {"gemm": 3.6484e9, "normmap": 1.6115e9, "normmap_a_pruned": 1.3043e9, "normmap_b_pruned": 1.3915e9},
 }
 
 WORKLOADS = {
@@ -104,8 +104,8 @@ def cpu_baseline(A, B, tile, tau, budget_s):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-literal", action="store_true", help="skip the one-off run of the literal lam=0.1 config")
