@@ -292,3 +292,37 @@ def test_stage_api_equals_multiply(orc, ctx):
     ctx.gemm_gated(C2)
     C3 = ctx.multiply(dA, dB, 64, 0.0)
     assert torch.equal(C2, C3)
+
+
+def test_two_contexts_on_two_streams_do_not_interfere(orc, ctx):
+    """Distinct contexts are independent (no globals): two of them, each on its own stream (default
+    priority), run different problems alternately; each must reproduce what the session context
+    computes alone."""
+    import torch
+    import cuspamm_amd as sp
+    cases = []
+    for M, K, N, tile, lam, ratio, seed in [(768, 512, 640, 64, 0.01, 0.3, 5), (512, 1024, 384, 32, 0.02, 0.1, 7)]:
+        tab = orc.decay_table("exp", max(M, K, N), lam)
+        dA, dB = _dev(orc.fill_decay(M, K, tab, seed)), _dev(orc.fill_decay(K, N, tab, seed + 1))
+        ctx.normmap_f32(1, dB, tile)
+        ctx.normmap_f32(0, dA, tile)
+        tau = ctx.tau_for_ratio(ratio)[0]
+        cases.append((dA, dB, tile, tau, ctx.multiply(dA, dB, tile, tau).clone(), ctx.get_mask()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    others = [sp.SpammContext(0), sp.SpammContext(0)]
+    outs = [torch.empty_like(c[4]) for c in cases]
+    try:
+        for c2, s in zip(others, streams):
+            c2.set_stream(s.cuda_stream)
+        for rep in range(4):
+            for i in (0, 1):
+                dA, dB, tile, tau = cases[i][:4]
+                others[i].multiply(dA, dB, tile, tau, C=outs[i], prune=bool(rep & 1))
+        for i in (0, 1):
+            others[i].synchronize()
+            assert torch.equal(outs[i], cases[i][4])
+            assert np.array_equal(others[i].get_mask(), cases[i][5])
+    finally:
+        for c2 in others:
+            c2.close()
