@@ -9,6 +9,10 @@ from .api import (  # noqa: F401
     ROLE_A,
     ROLE_B,
     FLAG_TIMING,
+    FLAG_A_EQ_B,
+    FLAG_REUSE_A,
+    FLAG_REUSE_B,
+    FLAG_PRUNE,
     SpammContext,
     SpammError,
     SpammParams,

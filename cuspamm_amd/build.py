@@ -65,7 +65,9 @@ def build_library(verbose=False):
 
     def compile_one(pair):
         src, obj = pair
-        extra = ["-Rpass-analysis=kernel-resource-usage"] if src == "kernels_gemm.hip" else []
+        # kernels_gemm.hip lists M0 as clobbered by its global->LDS loads; clang remarks on every
+        # instance that M0 is a reserved register (it never allocates it anyway): silenced there
+        extra = ["-Rpass-analysis=kernel-resource-usage", "-Wno-inline-asm"] if src == "kernels_gemm.hip" else []
         log = _run([HIPCC] + CFLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
         if extra:
             _check_no_scratch(log, src)

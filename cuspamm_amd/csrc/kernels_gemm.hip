@@ -56,13 +56,14 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // LDS write it cannot disambiguate (it would put a full vmcnt(0) wait before
 // every LDS read and serialise the staging ring); completion is awaited
 // explicitly with s_waitcnt vmcnt before the workgroup barrier.  M0 carries
-// the LDS address; nothing else in this kernel keeps a value in M0.
+// the LDS address and is declared clobbered, so the compiler keeps nothing
+// live in it across a load.
 template <int IMM>
 __device__ __forceinline__ void dma_load(const unsigned char *sbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(sbase), "n"(IMM)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // One workgroup per macro tile.  The k loop walks stages of 32 k (a list entry
@@ -209,7 +210,15 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         };
         auto issue_head = [&](const StageAddr &sa) { SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); };
         // every wave: own loads of the next stage landed and own LDS reads
-        // done; then the barrier makes both true for the whole workgroup
+        // done; then the barrier makes both true for the whole workgroup.
+        // INVARIANT behind the hand-counted vmcnt: between the prologue and
+        // the end of loop 2 the only vector-memory operations a wave issues
+        // are the LPW dma_loads per stage, in stage order (entries and k come
+        // through scalar loads, operands through LDS reads, C is stored after
+        // the loops).  vmcnt counts completions in issue order, so "at most
+        // LPW * (NBUF - 2) outstanding" means every load of the next stage
+        // has landed.  Any other global load or store added inside the loops
+        // breaks this count: re-derive it.
         auto sync_next = [&]() {
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2), 0));
             __syncthreads();

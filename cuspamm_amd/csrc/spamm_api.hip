@@ -33,6 +33,8 @@ struct spamm_ctx {
     int64_t M = 0, K = 0, N = 0;
     int tile = 0;
     bool have_a = false, have_b = false, have_gate = false;
+    // nA / nB+nBt hold norm maps of the current M x K / K x N at the current tile
+    bool nm_a = false, nm_b = false;
     float tau = 0.0f;
     // A's fp16 copy was written by a tau-aware pass: tiles that no product can keep at
     // a_pruned_tau are missing, so the copy serves a GEMM only for tau >= a_pruned_tau
@@ -120,6 +122,7 @@ void reset_shape(spamm_ctx *c, int tile) {
     c->tile = tile;
     c->M = c->K = c->N = 0;
     c->have_a = c->have_b = c->have_gate = false;
+    c->nm_a = c->nm_b = false;
     c->a_pruned = c->b_pruned = false;
 }
 
@@ -217,9 +220,13 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
     if (rc) return rc;
     if (c->tile != tile) reset_shape(c, tile);
     const size_t nt = (size_t)(rows / tile) * (size_t)(cols / tile);
+    c->have_gate = false;
     if (role == SPAMM_ROLE_A) {
-        // a new A invalidates B only if the shared dimension K changes
-        if (c->have_b && c->K != cols) c->have_b = false;
+        // a new A invalidates B (fp16 copy and norm map alike) only if the shared dimension K
+        // changes; A itself is invalid until its pass has been launched
+        if (c->K != cols) c->have_b = c->nm_b = false;
+        c->have_a = c->nm_a = false;
+        c->a_pruned = false;
         c->M = rows;
         c->K = cols;
         if ((rc = ensure(c, c->packedA, (size_t)rows * cols * 2))) return rc;
@@ -234,12 +241,14 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
         HIPCHK(c, launch_normmap_a(dX, in16, rows, cols, tile, c->packedA.p, (float *)c->nA.p,
                                    prune ? (const float *)c->rowmaxB.p : nullptr, prune ? *prune_tau : 0.0f, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[2], c->stream)); c->ev_a = true; }
-        c->have_a = true;
+        c->have_a = c->nm_a = true;
         c->a_pruned = prune;
         c->a_pruned_tau = prune ? *prune_tau : 0.0f;
     } else {
-        if (c->have_a && c->K != rows) c->have_a = false;
+        if (c->K != rows) c->have_a = c->nm_a = false;
         if (c->a_pruned) c->have_a = false;     // pruned against the previous B's norms
+        c->have_b = c->nm_b = false;
+        c->b_pruned = false;
         c->K = rows;
         c->N = cols;
         if ((rc = ensure(c, c->packedB, (size_t)rows * cols * 2))) return rc;
@@ -250,10 +259,9 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
         HIPCHK(c, launch_normmap_b(dX, in16, rows, cols, tile, c->packedB.p, (float *)c->nB.p,
                                    (float *)c->nBt.p, prune ? *prune_tau : 0.0f, c->stream));
         if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[1], c->stream)); c->ev_b = true; }
-        c->have_b = true;
+        c->have_b = c->nm_b = true;
         c->b_pruned = prune;
     }
-    c->have_gate = false;
     return SPAMM_OK;
 }
 
@@ -287,18 +295,20 @@ int spamm_set_normmaps(spamm_ctx *c, const float *nA, const float *nB, int64_t n
     HIPCHK(c, hipStreamSynchronize(c->stream));
     // norm maps only: the gate may run, the GEMM may not (no operands)
     c->have_a = c->have_b = false;
+    c->nm_a = c->nm_b = true;
     c->have_gate = false;
     return SPAMM_OK;
 }
 
 int spamm_gate(spamm_ctx *c, float tau) {
     if (!c) return SPAMM_EINVAL;
-    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     if (tau != tau) return SPAMM_EINVAL;   // NaN
     int rc = set_device(c);
     if (rc) return rc;
     const Shape s = shape_of(c);
     if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // K / tile beyond ~19 500 (tile 32)
+    if (order_lds_bytes(c->tile, s.nbM, s.nbN) > order_lds_limit()) return SPAMM_EINVAL;   // more than 8192 super tiles of C
     const size_t nt = (size_t)s.nbM * s.nbN;
     if ((rc = ensure(c, c->counts, nt * 4))) return rc;
     if ((rc = ensure(c, c->mask, nt * s.words * 8))) return rc;
@@ -359,6 +369,10 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
         if (n / p->tile > 65535) return SPAMM_EINVAL;
         if ((rc = set_device(c))) return rc;
         const size_t nt = (size_t)(n / p->tile) * (size_t)(n / p->tile);
+        // nothing of the old contents is valid until the pass has been launched
+        c->have_a = c->have_b = c->have_gate = false;
+        c->nm_a = c->nm_b = false;
+        c->a_pruned = c->b_pruned = false;
         if ((rc = ensure(c, c->packedA, (size_t)n * n * 2))) return rc;
         if ((rc = ensure(c, c->packedB, (size_t)n * n * 2))) return rc;
         if ((rc = ensure(c, c->nA, nt * 4))) return rc;
@@ -375,6 +389,7 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
             c->ev_a = c->ev_b = true;
         }
         c->have_a = c->have_b = true;
+        c->nm_a = c->nm_b = true;
         c->a_pruned = c->b_pruned = prune;       // both copies lack their tiles of norm zero:
         c->a_pruned_tau = 1.0e-45f;              // they serve any tau > 0 (smallest positive float)
         c->have_gate = false;
@@ -428,7 +443,7 @@ int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_
 int spamm_dropped_bound(spamm_ctx *c, float tau, double *out) {
     if (!c || !out || tau != tau) return SPAMM_EINVAL;
     Shape s;
-    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     int rc = set_device(c);
     if (rc) return rc;
     s = shape_of(c);
@@ -551,7 +566,7 @@ int spamm_load_mtx_f32(const char *path, int64_t rows, int64_t cols, int64_t ld,
 }
 
 static int tau_prepare(spamm_ctx *c, Shape *s) {
-    if (!c->tile || !c->M || !c->K || !c->N || !c->nA.p || !c->nBt.p) return SPAMM_ESTATE;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     int rc = set_device(c);
     if (rc) return rc;
     *s = shape_of(c);
@@ -661,11 +676,11 @@ int spamm_get_normmap(spamm_ctx *c, int role, float *host_out) {
     if (!c->tile) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
     if (role == SPAMM_ROLE_A) {
-        if (!c->nA.p || !c->M || !c->K) return SPAMM_ESTATE;
+        if (!c->nm_a) return SPAMM_ESTATE;
         return copy_out(c, c->nA.p, host_out, (size_t)s.nbM * s.nbK * 4);
     }
     if (role == SPAMM_ROLE_B) {
-        if (!c->nB.p || !c->K || !c->N) return SPAMM_ESTATE;
+        if (!c->nm_b) return SPAMM_ESTATE;
         return copy_out(c, c->nB.p, host_out, (size_t)s.nbK * s.nbN * 4);
     }
     return SPAMM_EINVAL;

@@ -92,6 +92,13 @@ hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *
 
 size_t gate_lds_bytes(int tile, int64_t nbK);
 inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k_gate (a few static bytes aside)
+// k_order ranks the super tiles of C (4 x 8 macro tiles of 256 x 256) in one workgroup's LDS
+inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
+    const int MT = 256 / tile;
+    const int64_t nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
+    return (size_t)(((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N)) * 2 * sizeof(int);
+}
+inline size_t order_lds_limit() { return 64 * 1024; }
 hipError_t gate_init();   // one-time kernel attribute set-up
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
                        float tau, hipStream_t s);

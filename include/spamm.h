@@ -124,7 +124,9 @@ SPAMM_API int spamm_normmap_f16(spamm_ctx *ctx, int role, const void *dXh, int64
  * (cuSpAMM.cu:302-334): per output tile the kept-k bitmap and the count (the
  * ascending compacted k list of :315-325 is the bitmap's set bits in order;
  * spamm_get_klist materialises it).  Uses the norm maps left by stage 1 (or by
- * spamm_set_normmaps). */
+ * spamm_set_normmaps); SPAMM_ESTATE unless both are present for the same K and tile.
+ * Shape limits (SPAMM_EINVAL): K / tile up to about 19 500 at tile 32 (a macro tile's bitmaps are
+ * held in LDS; far more at tile 64 / 128), and at most 8192 super tiles of 1024 x 2048 elements of C. */
 SPAMM_API int spamm_gate(spamm_ctx *ctx, float tau);
 
 /* Stage 3 -- replaces the product loop of get_C_FP16_B32 (cuSpAMM.cu:336-391):

@@ -268,6 +268,37 @@ def test_argument_errors(ctx):
     fresh.close()
 
 
+def test_stages_refuse_norm_maps_of_mismatched_shape(ctx):
+    """A norm map of B taken at one K and one of A taken at another must not be gated together:
+    every stage that reads both returns SPAMM_ESTATE (and launches nothing)."""
+    import torch
+    import cuspamm_amd as sp
+    fresh = sp.SpammContext(0)
+    B = torch.ones((128, 128), dtype=torch.float32, device="cuda")
+    A = torch.ones((128, 256), dtype=torch.float32, device="cuda")
+    fresh.normmap_f32(sp.ROLE_B, B, 32)                       # K = 128
+    fresh.normmap_f32(sp.ROLE_A, A, 32)                       # K = 256: B's map no longer fits
+    for call in (lambda: fresh.gate(0.0), lambda: fresh.tau_for_ratio(0.5), lambda: fresh.count_kept(0.0),
+                 lambda: fresh.dropped_bound(0.0), lambda: fresh.tune_bisect(), lambda: fresh.get_normmap(sp.ROLE_B)):
+        with pytest.raises(sp.SpammError) as ei:
+            call()
+        assert ei.value.code == -4
+    assert fresh.get_normmap(sp.ROLE_A).shape == (4, 8)       # A's own map is fine
+    fresh.normmap_f32(sp.ROLE_B, torch.ones((256, 64), dtype=torch.float32, device="cuda"), 32)
+    fresh.gate(0.0)                                           # matching K again
+    assert int(fresh.get_counts().sum()) == 4 * 8 * 2
+    # the other way round, and a tile change
+    fresh.normmap_f32(sp.ROLE_B, B, 32)
+    with pytest.raises(sp.SpammError) as ei:
+        fresh.gate(0.0)
+    assert ei.value.code == -4
+    fresh.normmap_f32(sp.ROLE_A, torch.ones((64, 128), dtype=torch.float32, device="cuda"), 64)
+    with pytest.raises(sp.SpammError) as ei:
+        fresh.gate(0.0)
+    assert ei.value.code == -4
+    fresh.close()
+
+
 def test_workspace_reuse_across_shapes(orc, ctx):
     # same context, shrinking and growing problems, different tiles: no stale state
     for M, K, N, tile, tau in [(512, 256, 384, 64, 5.0), (128, 128, 128, 32, 0.1), (768, 512, 256, 128, 100.0),

@@ -10,6 +10,20 @@ def _dev(x):
     return torch.from_numpy(np.ascontiguousarray(x)).cuda()
 
 
+def _vs_checker(orc, ctx, C, A32, B32, tile, tau, what):
+    """The library's last multiply against the host checker run on the same fp32 values: kept mask,
+    counts and norm maps bit-exact, C within 1e-3 relative Frobenius error."""
+    ref = orc.spamm(np.ascontiguousarray(A32, dtype=np.float32), np.ascontiguousarray(B32, dtype=np.float32), tile, tau)
+    assert np.array_equal(ctx.get_mask(), ref["mask"]), what
+    assert np.array_equal(ctx.get_counts(), ref["counts"]), what
+    assert np.array_equal(ctx.get_normmap(0).view(np.uint32), ref["nA"].view(np.uint32)), what
+    assert np.array_equal(ctx.get_normmap(1).view(np.uint32), ref["nB"].view(np.uint32)), what
+    assert ctx.get_stats().kept_products == ref["kept"], what
+    err, nrm, _ = orc.frob_diff(C.cpu().numpy(), ref["C"])
+    assert err <= 1e-3 * nrm, "%s: C off by %g" % (what, err / max(nrm, 1e-300))
+    return ref
+
+
 @pytest.mark.parametrize("tile", [32, 64, 128])
 def test_fp16_inputs_equal_fp32_inputs_of_the_same_values(orc, ctx, tile):
     import torch
@@ -22,6 +36,9 @@ def test_fp16_inputs_equal_fp32_inputs_of_the_same_values(orc, ctx, tile):
     tau, ach = ctx.tau_for_ratio(0.5)
     assert 0.45 < ach < 0.6
     C16 = ctx.multiply(A, B, tile, tau).clone()
+    # fp16 is the reference's real input type (para.h:1, cuSpAMM.cu:486): the checker, fed the same
+    # values as fp32 (its fp16 rounding is then the identity), must agree
+    _vs_checker(orc, ctx, C16, A.float().cpu().numpy(), B.float().cpu().numpy(), tile, tau, "fp16 inputs")
     m16, nA16, nB16 = ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1)
     assert np.array_equal(ctx.get_fp16(0), A.cpu().numpy().view(np.uint16))
     assert np.array_equal(ctx.get_fp16(1), B.cpu().numpy().view(np.uint16))
@@ -30,7 +47,9 @@ def test_fp16_inputs_equal_fp32_inputs_of_the_same_values(orc, ctx, tile):
     assert np.array_equal(ctx.get_normmap(0).view(np.uint32), nA16.view(np.uint32))
     assert np.array_equal(ctx.get_normmap(1).view(np.uint32), nB16.view(np.uint32))
     assert torch.equal(C16, C32)
-    assert torch.equal(C16, ctx.multiply(A, B, tile, tau, prune=True))      # tau-aware passes on fp16 inputs
+    Cp = ctx.multiply(A, B, tile, tau, prune=True)      # tau-aware passes on fp16 inputs
+    assert torch.equal(C16, Cp)
+    _vs_checker(orc, ctx, Cp, A.float().cpu().numpy(), B.float().cpu().numpy(), tile, tau, "fp16 inputs, tau-aware")
     kept = ctx.get_stats().kept_products
     assert 0 < kept < (M // tile) * (K // tile) * (N // tile)
 
@@ -44,12 +63,21 @@ def test_operand_reuse(orc, ctx):
     ref1 = ctx.multiply(A1, B, 64, 0.5).clone()
     ref2 = ctx.multiply(A2, B, 64, 0.5).clone()
     ctx.multiply(A1, B, 64, 0.5)
+    hA1, hA2, hB = A1.cpu().numpy(), A2.cpu().numpy(), B.cpu().numpy()
     got2 = ctx.multiply(A2, B, 64, 0.5, reuse_b=True)          # B's fp16 copy and norm map are kept
     assert torch.equal(got2, ref2)
+    _vs_checker(orc, ctx, got2, hA2, hB, 64, 0.5, "new A against the resident B")
     got1 = ctx.multiply(A1, B, 64, 0.5, reuse_b=True)
     assert torch.equal(got1, ref1)
+    _vs_checker(orc, ctx, got1, hA1, hB, 64, 0.5, "first A again against the resident B")
     got1 = ctx.multiply(A1, B, 64, 0.1, reuse_a=True, reuse_b=True)   # only tau changes
-    assert torch.equal(got1, ctx.multiply(A1, B, 64, 0.1))
+    _vs_checker(orc, ctx, got1, hA1, hB, 64, 0.1, "both operands resident, new tau")
+    assert torch.equal(got1.clone(), ctx.multiply(A1, B, 64, 0.1))
+    # a new B against the resident A (matrix powers: X, then X * B2)
+    B2 = _dev(orc.fill_decay(n, n, tab, 9))
+    ctx.multiply(A1, B, 64, 0.5)
+    gotb = ctx.multiply(A1, B2, 64, 0.5, reuse_a=True)
+    _vs_checker(orc, ctx, gotb, hA1, B2.cpu().numpy(), 64, 0.5, "new B against the resident A")
     with pytest.raises(sp.SpammError) as ei:                    # shape changed: nothing to reuse
         ctx.multiply(A1[:256].contiguous(), B, 64, 0.5, reuse_a=True)
     assert ei.value.code == -4
@@ -91,6 +119,9 @@ def test_a_equals_b_single_pass(orc, ctx, tile):
     C2 = ctx.multiply(X, X, tile, tau).clone()
     ref = (ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1), ctx.get_fp16(0), ctx.get_fp16(1))
     C1 = ctx.multiply(X, X, tile, tau, a_eq_b=True)
+    hX = X.cpu().numpy()
+    chk = _vs_checker(orc, ctx, C1, hX, hX, tile, tau, "A = B single pass")
+    assert np.array_equal(ctx.get_fp16(0), chk["hA"]) and np.array_equal(ctx.get_fp16(1), chk["hB"])
     got = (ctx.get_mask(), ctx.get_normmap(0), ctx.get_normmap(1), ctx.get_fp16(0), ctx.get_fp16(1))
     for r, g in zip(ref, got):
         assert np.array_equal(r.view(np.uint8), g.view(np.uint8))
@@ -103,8 +134,10 @@ def test_a_equals_b_single_pass(orc, ctx, tile):
     # (exp(-0.5 d) is exactly zero in fp16 beyond d = 33, exp(-0.05 d) beyond d = 333)
     assert np.count_nonzero(ref[1] == 0) > 0
     ctx.multiply(torch.full_like(X, 1000.0), X, tile, 0.0)   # loud workspace
-    assert torch.equal(ctx.multiply(X, X, tile, tau, a_eq_b=True, prune=True), C2)
+    Cp = ctx.multiply(X, X, tile, tau, a_eq_b=True, prune=True)
+    assert torch.equal(Cp, C2)
     assert np.array_equal(ctx.get_mask(), ref[0])
+    _vs_checker(orc, ctx, Cp, hX, hX, tile, tau, "A = B single pass, tau-aware")
     with pytest.raises(sp.SpammError):
         ctx.get_fp16(0)
     with pytest.raises(sp.SpammError):
