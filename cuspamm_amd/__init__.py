@@ -13,6 +13,7 @@ from .api import (  # noqa: F401
     FLAG_REUSE_A,
     FLAG_REUSE_B,
     FLAG_PRUNE,
+    NOALLOC_WORKSPACE_BYTES,
     SpammContext,
     SpammError,
     SpammParams,

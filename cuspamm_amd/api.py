@@ -19,7 +19,8 @@ FLAG_REUSE_A = 4
 FLAG_REUSE_B = 8
 FLAG_PRUNE = 16
 
-OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV = 0, -1, -2, -3, -4, -5
+OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV, ELIMIT = 0, -1, -2, -3, -4, -5, -6
+NOALLOC_WORKSPACE_BYTES = 40 << 20
 
 
 class SpammParams(ctypes.Structure):
@@ -68,6 +69,7 @@ def load_library():
     L.spamm_destroy.argtypes = [vp]
     L.spamm_set_stream.argtypes = [vp, vp]
     L.spamm_multiply.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
+    L.spamm_multiply_noalloc.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
     L.spamm_normmap_f32.argtypes = [vp, ctypes.c_int, vp, i64, i64, i32]
     L.spamm_normmap_f16.argtypes = [vp, ctypes.c_int, vp, i64, i64, i32]
     L.spamm_multiply_f16.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
@@ -196,6 +198,21 @@ class SpammContext:
             _check(self._lib.spamm_multiply(self._h, ctypes.byref(p), _devptr(A, "float32"),
                                             _devptr(B, "float32"), _devptr(C, "float32")),
                    "spamm_multiply")
+        self._shape = (M // tile, K // tile, N // tile, int(tile), M, K, N)
+        return C
+
+    def multiply_noalloc(self, A, B, tile, tau, C, timing=False, a_eq_b=False, prune=False):
+        """spamm_multiply_noalloc: the same multiply in the library's fixed device workspace (fp32 inputs,
+        caller-provided C, no device allocation inside the call; SpammError ELIMIT beyond the workspace)."""
+        M, K = A.shape
+        K2, N = B.shape
+        if K != K2:
+            raise ValueError("inner dimensions differ")
+        flags = (FLAG_TIMING if timing else 0) | (FLAG_A_EQ_B if a_eq_b else 0) | (FLAG_PRUNE if prune else 0)
+        p = SpammParams(M, K, N, int(tile), float(tau), flags, 0)
+        _check(self._lib.spamm_multiply_noalloc(self._h, ctypes.byref(p), _devptr(A, "float32"),
+                                                _devptr(B, "float32"), _devptr(C, "float32")),
+               "spamm_multiply_noalloc")
         self._shape = (M // tile, K // tile, N // tile, int(tile), M, K, N)
         return C
 

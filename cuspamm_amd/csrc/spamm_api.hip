@@ -5,6 +5,7 @@
 
 #include <math.h>
 #include <new>
+#include <utility>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -14,21 +15,27 @@
 
 using namespace spamm;
 
+// Workspace of spamm_multiply_noalloc: one fixed array per GPU, part of the code object, held from
+// the moment the library is loaded until the process ends.  In host code this name is only a
+// handle for hipGetSymbolAddress: the device address is looked up once per context (= per device)
+// in spamm_create and everything below uses that pointer.
+static __device__ __align__(256) unsigned char scratch[SPAMM_NOALLOC_WORKSPACE_BYTES];
+
 namespace {
 
 struct DevBuf {
     void *p = nullptr;
     size_t cap = 0;
+    bool borrowed = false;    // p points into the fixed device array: never freed
 };
 
 }  // namespace
 
-struct spamm_ctx {
-    int device = 0;
-    hipStream_t own_stream = nullptr;
-    hipStream_t stream = nullptr;
-    int last_hip = 0;
-
+// Everything a multiply leaves behind: the shape it ran at, what is valid, and
+// the device buffers.  A context holds two of these: its own (hipMalloc'd, grown
+// on demand) and one carved out of the library's fixed device array for
+// spamm_multiply_noalloc; `static_cast<Workspace &>(*ctx)` is the live one.
+struct Workspace {
     // problem shape of the current workspace contents
     int64_t M = 0, K = 0, N = 0;
     int tile = 0;
@@ -45,7 +52,20 @@ struct spamm_ctx {
 
     DevBuf packedA, packedB, nA, nB, nBt, rowmaxB;
     DevBuf counts, klist, mask, macro_list, macro_count, macro_work, order, sched, kept_total;
-    DevBuf scratch;   // read-back staging / decay table
+};
+
+struct spamm_ctx : Workspace {
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    int last_hip = 0;
+
+    Workspace parked;           // the workspace that is not live (see in_static)
+    bool in_static = false;     // live workspace = carve-outs of the fixed device array
+    bool no_alloc = false;      // inside spamm_multiply_noalloc: ensure() must not allocate
+    unsigned char *static_ptr = nullptr;   // device address of the fixed array on this context's device
+
+    DevBuf staging;   // read-back staging / decay table
     DevBuf tauws;     // tau selection workspace
 
     hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -68,12 +88,14 @@ namespace {
 int ensure(spamm_ctx *c, DevBuf &b, size_t bytes) {
     if (bytes == 0) bytes = 16;
     if (b.cap >= bytes) return SPAMM_OK;
-    if (b.p) {
+    if (c->no_alloc) return SPAMM_ELIMIT;       // the carve-out was sized by the same formulas: not reached
+    if (b.p && !b.borrowed) {
         HIPCHK(c, hipStreamSynchronize(c->stream));
         HIPCHK(c, hipFree(b.p));
-        b.p = nullptr;
-        b.cap = 0;
     }
+    b.p = nullptr;
+    b.cap = 0;
+    b.borrowed = false;
     HIPCHK(c, hipMalloc(&b.p, bytes));
     b.cap = bytes;
     return SPAMM_OK;
@@ -126,6 +148,25 @@ void reset_shape(spamm_ctx *c, int tile) {
     c->a_pruned = c->b_pruned = false;
 }
 
+// The buffers of a workspace that the library allocated (carve-outs of the fixed array are not freed).
+void free_workspace(Workspace &w) {
+    DevBuf *bufs[] = {&w.packedA, &w.packedB, &w.nA, &w.nB, &w.nBt, &w.rowmaxB, &w.counts, &w.klist,
+                      &w.mask, &w.macro_list, &w.macro_count, &w.macro_work, &w.order, &w.sched, &w.kept_total};
+    for (DevBuf *b : bufs) {
+        if (b->p && !b->borrowed) (void)hipFree(b->p);
+        *b = DevBuf();
+    }
+}
+
+// An ordinary producing call (multiply, norm-map stage, uploaded norm maps) works in the context's
+// own workspace: if the last call was spamm_multiply_noalloc, bring it back.  Its contents and
+// validity flags are as the last ordinary call left them.
+void leave_static(spamm_ctx *c) {
+    if (!c->in_static || c->no_alloc) return;
+    std::swap(static_cast<Workspace &>(*c), c->parked);
+    c->in_static = false;
+}
+
 int copy_out(spamm_ctx *c, const void *dev, void *host, size_t bytes) {
     HIPCHK(c, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
@@ -146,6 +187,7 @@ const char *spamm_strerror(int code) {
         case SPAMM_EHIP: return "HIP runtime error (see spamm_last_hip_error)";
         case SPAMM_ESTATE: return "stage called before the stage it depends on";
         case SPAMM_ENODEV: return "no usable gfx950 device";
+        case SPAMM_ELIMIT: return "problem needs more than the fixed workspace of spamm_multiply_noalloc";
         default: return "unknown error";
     }
 }
@@ -171,6 +213,12 @@ int spamm_create(spamm_ctx **out, int device) {
     for (int i = 0; i < 5 && rc == SPAMM_OK; i++)
         if (hipEventCreate(&c->ev[i]) != hipSuccess) rc = SPAMM_EHIP;
     if (rc == SPAMM_OK && (gemm_init() != hipSuccess || gate_init() != hipSuccess)) rc = SPAMM_EHIP;
+    if (rc == SPAMM_OK) {
+        // this device's copy of the fixed workspace array (each GPU has its own, at its own address)
+        void *sp = nullptr;
+        if (hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) != hipSuccess || !sp) rc = SPAMM_EHIP;
+        c->static_ptr = (unsigned char *)sp;
+    }
     if (rc != SPAMM_OK) {
         (void)hipGetLastError();
         spamm_destroy(c);          // releases whatever was created
@@ -184,11 +232,10 @@ int spamm_destroy(spamm_ctx *c) {
     if (!c) return SPAMM_EINVAL;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    DevBuf *bufs[] = {&c->packedA, &c->packedB, &c->nA, &c->nB, &c->nBt, &c->rowmaxB, &c->counts, &c->klist,
-                      &c->mask, &c->macro_list, &c->macro_count, &c->macro_work, &c->order,
-                      &c->sched, &c->kept_total, &c->scratch, &c->tauws};
-    for (DevBuf *b : bufs)
-        if (b->p) (void)hipFree(b->p);
+    free_workspace(*c);
+    free_workspace(c->parked);
+    if (c->staging.p) (void)hipFree(c->staging.p);
+    if (c->tauws.p) (void)hipFree(c->tauws.p);
     for (int i = 0; i < 5; i++)
         if (c->ev[i]) (void)hipEventDestroy(c->ev[i]);
     if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
@@ -218,6 +265,7 @@ static int normmap_any(spamm_ctx *c, int role, const void *dX, bool in16, int64_
     if (rows / tile > 65535 || cols / tile > 65535) return SPAMM_EINVAL;
     int rc = set_device(c);
     if (rc) return rc;
+    leave_static(c);
     if (c->tile != tile) reset_shape(c, tile);
     const size_t nt = (size_t)(rows / tile) * (size_t)(cols / tile);
     c->have_gate = false;
@@ -282,6 +330,7 @@ int spamm_set_normmaps(spamm_ctx *c, const float *nA, const float *nB, int64_t n
         return SPAMM_EINVAL;
     int rc = set_device(c);
     if (rc) return rc;
+    leave_static(c);
     reset_shape(c, tile);
     c->M = nbM * tile;
     c->K = nbK * tile;
@@ -349,6 +398,7 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     if (p->M <= 0 || p->K <= 0 || p->N <= 0) return SPAMM_EINVAL;
     if (p->M % p->tile || p->K % p->tile || p->N % p->tile) return SPAMM_EINVAL;
     if (p->tau != p->tau) return SPAMM_EINVAL;
+    leave_static(c);
     c->timing = (p->flags & SPAMM_FLAG_TIMING) != 0;
     c->ev_a = c->ev_b = c->ev_gate = c->ev_gemm = false;
     int rc;
@@ -415,6 +465,65 @@ static int multiply_any(spamm_ctx *c, const spamm_params *p, const void *dA, con
     return SPAMM_OK;
 }
 
+// Gives every buffer a multiply of this shape needs its place in the fixed array (base != null) and
+// returns the bytes used; with base == null only the size is computed.  Same sizes as the ensure()
+// calls of the stages.
+static size_t carve_static(Workspace &w, const spamm_params *p, unsigned char *base) {
+    const size_t t = (size_t)p->tile;
+    const size_t M = (size_t)p->M, K = (size_t)p->K, N = (size_t)p->N;
+    const size_t nbM = M / t, nbK = K / t, nbN = N / t, nt = nbM * nbN, words = (nbK + 63) / 64;
+    const size_t MT = (size_t)macro_dim(p->tile);
+    const size_t n_macro = ((nbM + MT - 1) / MT) * ((nbN + MT - 1) / MT);
+    size_t off = 0;
+    auto take = [&](DevBuf &b, size_t bytes) {
+        if (bytes == 0) bytes = 16;
+        if (base) {
+            if (b.p && !b.borrowed) (void)hipFree(b.p);    // not reached: the static workspace owns nothing here
+            b.p = base + off;
+            b.cap = bytes;
+            b.borrowed = true;
+        }
+        off += (bytes + 255) & ~(size_t)255;
+    };
+    take(w.packedA, M * K * 2);
+    take(w.packedB, K * N * 2);
+    take(w.nA, nbM * nbK * 4);
+    take(w.nB, nbK * nbN * 4);
+    take(w.nBt, nbK * nbN * 4);
+    take(w.rowmaxB, nbK * 4);
+    take(w.counts, nt * 4);
+    take(w.mask, nt * words * 8);
+    take(w.macro_list, n_macro * nbK * sizeof(MacroEntry));
+    take(w.macro_count, n_macro * 8);
+    take(w.macro_work, n_macro * 4);
+    take(w.order, (size_t)sched_rounds(p->tile, (int64_t)nbM, (int64_t)nbN) * NUM_XCD * SUPER_M * SUPER_N * 4);
+    take(w.sched, 2 * NUM_XCD * 4);
+    take(w.kept_total, 16);
+    return off;
+}
+
+int spamm_multiply_noalloc(spamm_ctx *c, const spamm_params *p, const float *dA, const float *dB, float *dC) {
+    if (!c || !p || !dA || !dB || !dC) return SPAMM_EINVAL;
+    if (p->flags & (SPAMM_FLAG_REUSE_A | SPAMM_FLAG_REUSE_B)) return SPAMM_EINVAL;   // the array is shared: nothing persists
+    if (!tile_ok(p->tile)) return SPAMM_EINVAL;
+    if (p->M <= 0 || p->K <= 0 || p->N <= 0) return SPAMM_EINVAL;
+    if (p->M % p->tile || p->K % p->tile || p->N % p->tile) return SPAMM_EINVAL;
+    if (p->M / p->tile > 65535 || p->K / p->tile > 65535 || p->N / p->tile > 65535) return SPAMM_ELIMIT;
+    if (p->tau != p->tau) return SPAMM_EINVAL;
+    if (!c->static_ptr) return SPAMM_ESTATE;
+    if (carve_static(*c, p, nullptr) > (size_t)SPAMM_NOALLOC_WORKSPACE_BYTES) return SPAMM_ELIMIT;
+    if (!c->in_static) {
+        std::swap(static_cast<Workspace &>(*c), c->parked);
+        c->in_static = true;
+    }
+    reset_shape(c, p->tile);           // the carve-outs move with the shape, and other contexts share the array
+    (void)carve_static(*c, p, c->static_ptr);
+    c->no_alloc = true;
+    const int rc = multiply_any(c, p, dA, dB, false, dC);
+    c->no_alloc = false;
+    return rc;
+}
+
 int spamm_multiply(spamm_ctx *c, const spamm_params *p, const float *dA, const float *dB, float *dC) {
     return multiply_any(c, p, dA, dB, false, dC);
 }
@@ -472,8 +581,8 @@ int spamm_mfma_ceiling(spamm_ctx *c, int random_operands, int iters, double *tfl
         h[i] = random_operands ? (_Float16)(((float)(x >> 8) / 8388608.0f) - 1.0f) : (_Float16)0.0f;
     }
     const size_t in_bytes = h.size() * 2, out_bytes = (size_t)n_wg * 256 * 4, tr_bytes = (size_t)n_wg * 16;
-    if ((rc = ensure(c, c->scratch, in_bytes + out_bytes + tr_bytes))) return rc;
-    char *base = (char *)c->scratch.p;
+    if ((rc = ensure(c, c->staging, in_bytes + out_bytes + tr_bytes))) return rc;
+    char *base = (char *)c->staging.p;
     HIPCHK(c, hipMemcpyAsync(base, h.data(), in_bytes, hipMemcpyHostToDevice, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
     double best_ns = 0.0, best_clk = 0.0;
@@ -729,9 +838,9 @@ int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
         return SPAMM_EINVAL;
     }
     const size_t bytes = (size_t)rows * cols * 2;
-    if ((rc = ensure(c, c->scratch, bytes))) return rc;
-    HIPCHK(c, launch_unpack(packed, rows, cols, c->tile, role, (uint16_t *)c->scratch.p, c->stream));
-    return copy_out(c, c->scratch.p, host_out, bytes);
+    if ((rc = ensure(c, c->staging, bytes))) return rc;
+    HIPCHK(c, launch_unpack(packed, rows, cols, c->tile, role, (uint16_t *)c->staging.p, c->stream));
+    return copy_out(c, c->staging.p, host_out, bytes);
 }
 
 int spamm_fill_decay_f32(spamm_ctx *c, float *dX, int64_t rows, int64_t cols,
@@ -740,9 +849,9 @@ int spamm_fill_decay_f32(spamm_ctx *c, float *dX, int64_t rows, int64_t cols,
     int rc = set_device(c);
     if (rc) return rc;
     const int64_t n = rows > cols ? rows : cols;
-    if ((rc = ensure(c, c->scratch, (size_t)n * 4))) return rc;
-    HIPCHK(c, hipMemcpyAsync(c->scratch.p, host_table, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
-    HIPCHK(c, launch_fill_decay(dX, rows, cols, (const float *)c->scratch.p, seed, random, c->stream));
+    if ((rc = ensure(c, c->staging, (size_t)n * 4))) return rc;
+    HIPCHK(c, hipMemcpyAsync(c->staging.p, host_table, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, launch_fill_decay(dX, rows, cols, (const float *)c->staging.p, seed, random, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
     return SPAMM_OK;
 }

@@ -34,6 +34,7 @@ extern "C" {
 #define SPAMM_EHIP (-3)      /* a HIP call failed; see spamm_last_hip_error */
 #define SPAMM_ESTATE (-4)    /* stage called before the stage it depends on */
 #define SPAMM_ENODEV (-5)    /* no usable gfx950 device */
+#define SPAMM_ELIMIT (-6)    /* spamm_multiply_noalloc: the problem needs more than the fixed workspace */
 
 /* Operand roles for the norm-map stage. */
 #define SPAMM_ROLE_A 0       /* contraction along columns: A[M x K] */
@@ -109,6 +110,23 @@ SPAMM_API int spamm_multiply(spamm_ctx *ctx, const spamm_params *p, const float 
  * arrays.  The norm-map stage then only packs and takes norms. */
 SPAMM_API int spamm_multiply_f16(spamm_ctx *ctx, const spamm_params *p, const void *dAh, const void *dBh,
                                  float *dC);
+
+/* spamm_multiply for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * main() allocates everything up front (cuSpAMM.cu:435-439).  Same arguments, same result, but the
+ * whole workspace -- fp16 operand copies, norm maps, gate bitmaps and lists, schedule -- lives in one
+ * fixed device array of SPAMM_NOALLOC_WORKSPACE_BYTES that is part of the library image (every GPU
+ * the library runs on holds it until the process ends), and the call makes no hipMalloc / hipFree.
+ * Limit: the buffers for (M, K, N, tile) must fit the array -- 2(MK + KN) bytes of fp16 copies plus
+ * ~1 % for the rest, e.g. up to 2048 x 4096 x 2048 or 3072^3 -- else SPAMM_ELIMIT.
+ * SPAMM_FLAG_REUSE_A/B are rejected (SPAMM_EINVAL).  All contexts on one GPU share the array and it
+ * keeps the last call's contents: calls that overlap in time on one GPU (two contexts, two
+ * streams) race; issue them one after the other.  Afterwards the context's read-backs and stage
+ * calls refer to this call's results; the next ordinary multiply / norm-map call returns to the
+ * context's own workspace, whose contents (and REUSE state) are as it left them. */
+#define SPAMM_NOALLOC_WORKSPACE_BYTES (40u << 20)
+SPAMM_API int spamm_multiply_noalloc(spamm_ctx *ctx, const spamm_params *p, const float *dA, const float *dB,
+                                     float *dC);
 
 /* Stage 1 -- replaces unroll_get_Fnorm_FP16 / unroll_get_Fnorm_pri
  * (cuSpAMM.cu:74-123, 21-71; launches :478-503) plus the host fp16 conversion:

@@ -19,7 +19,7 @@ def test_header_declares_the_expected_entry_points():
     syms = _declared_symbols()
     for must in ("spamm_create", "spamm_destroy", "spamm_multiply", "spamm_normmap_f32", "spamm_gate",
                  "spamm_gemm_gated", "spamm_get_mask", "spamm_get_counts", "spamm_get_klist",
-                 "spamm_get_normmap", "spamm_strerror"):
+                 "spamm_get_normmap", "spamm_strerror", "spamm_multiply_noalloc"):
         assert must in syms
 
 
@@ -47,15 +47,23 @@ def test_flag_values_match_header():
         assert getattr(api, name) == int(value), name
 
 
+def test_noalloc_workspace_size_matches_header():
+    from cuspamm_amd import api
+    text = open(os.path.join(ROOT, "include", "spamm.h")).read()
+    m = re.search(r"#define\s+SPAMM_NOALLOC_WORKSPACE_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", text)
+    assert m and (int(m.group(1)) << int(m.group(2))) == api.NOALLOC_WORKSPACE_BYTES
+    assert api.ELIMIT == int(re.search(r"#define\s+SPAMM_ELIMIT\s+\((-\d+)\)", text).group(1))
+
+
 def test_error_strings():
     import cuspamm_amd as sp
     L = sp.load_library()
     seen = set()
-    for code in (0, -1, -2, -3, -4, -5):
+    for code in (0, -1, -2, -3, -4, -5, -6):
         s = L.spamm_strerror(code).decode()
         assert s and s != "unknown error"
         seen.add(s)
-    assert len(seen) == 6
+    assert len(seen) == 7
     assert L.spamm_strerror(-99).decode() == "unknown error"
 
 
@@ -66,6 +74,7 @@ def test_null_arguments_are_rejected_without_a_device():
     assert L.spamm_destroy(None) == -1
     assert L.spamm_gate(None, 0.0) == -1
     assert L.spamm_multiply(None, None, None, None, None) == -1
+    assert L.spamm_multiply_noalloc(None, None, None, None, None) == -1
 
 
 def test_create_without_gpu_reports_no_device():
