@@ -280,8 +280,9 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 
 // Schedule for the GEMM.  Macro tiles are grouped into super tiles of
 // SUPER_M x SUPER_N (= 32, one per CU of an XCD); workgroups are dispatched
-// round-robin over the 8 XCDs, so workgroup b runs on XCD b % 8 and is the
-// (b / 8)-th workgroup that XCD starts.
+// round-robin over the n_xcd XCDs of the device, so workgroup b runs on XCD
+// b % n_xcd and is the (b / n_xcd)-th workgroup that XCD starts (n_xcd = 1: one
+// flat sequence, for devices that are not whole XCDs of 32 CUs).
 //   1. Super tiles are ranked by descending kept-product count and dealt to
 //      the XCDs in snake order: every XCD owns whole super tiles, so the
 //      workgroups sharing one L2 share A row panels and B column panels, and
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // computing items, sched[8 + x] = number of all items.
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
-                                                int n_super, int rounds) {
+                                                int n_super, int rounds, int n_xcd) {
     extern __shared__ int swork[];               // [n_super] work, then [n_super] super tile origin by rank
     int *srank_id = swork + n_super;
     __shared__ unsigned long long total;
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     // macro tile of XCD x at raw position p (round-major, then slot inside the super tile), or -1
     auto macro_at = [&](int x, int p) -> int {
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
-        const int sr = round * NUM_XCD + ((round & 1) ? NUM_XCD - 1 - x : x);
+        const int sr = round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
         if (p >= P || sr >= n_super) return -1;
         const int origin = srank_id[sr];
         const int mi = (origin >> 16) + slot / SUPER_N, mj = (origin & 0xffff) + slot % SUPER_N;
@@ -342,7 +343,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     };
     // one wave per XCD: computing macro tiles to the front in raw order, empty ones from the back
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (wave < NUM_XCD) {
+    if (wave < n_xcd) {
         const int x = wave;
         int nall = 0;                            // macro tiles in this XCD's sequence (no memory access)
         for (int p0 = 0; p0 < P; p0 += 64) nall += __builtin_popcountll(__ballot(macro_at(x, p0 + lane) >= 0));
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         }
         if (lane == 0) {
             g.sched[x] = nc;
-            g.sched[NUM_XCD + x] = nall;
+            g.sched[MAX_XCD + x] = nall;
         }
     }
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;
@@ -416,7 +417,7 @@ hipError_t gate_init() {
 }
 
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
-                       float tau, hipStream_t s) {
+                       float tau, int n_xcd, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nMacM = (int)((nbM + MT - 1) / MT), nMacN = (int)((nbN + MT - 1) / MT);
     const int n_macro = nMacM * nMacN;
@@ -431,8 +432,8 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     if (e != hipSuccess) return e;
     const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
     const int n_super = nSupM * nSupN;
-    const int rounds = (n_super + NUM_XCD - 1) / NUM_XCD;
-    k_order<<<1, 1024, (size_t)n_super * 2 * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super, rounds);
+    const int rounds = (n_super + n_xcd - 1) / n_xcd;
+    k_order<<<1, 1024, (size_t)n_super * 2 * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super, rounds, n_xcd);
     return hipGetLastError();
 }
 

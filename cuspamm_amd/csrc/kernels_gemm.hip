@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
                                               const MacroEntry *__restrict__ macro_list,
                                               const int32_t *__restrict__ macro_count,
                                               const int32_t *__restrict__ order,
-                                              const int32_t *__restrict__ sched, int P, int nbM,
+                                              const int32_t *__restrict__ sched, int P, int n_xcd, int nbM,
                                               int nbK, int nbN, int nMacN, int64_t M, int64_t N,
                                               float *__restrict__ C) {
     using G = GemmCfg<B>;
@@ -88,14 +88,14 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
-    // Workgroup b runs on XCD b % NUM_XCD and is that XCD's q-th workgroup,
-    // q = b / NUM_XCD; `order` holds each XCD's sequence: computing macro tiles
+    // Workgroup b runs on XCD b % n_xcd and is that XCD's q-th workgroup,
+    // q = b / n_xcd; `order` holds each XCD's sequence: computing macro tiles
     // first, then the ones with nothing kept.  The latter's workgroups only
     // write zeros; they are dispatched when CUs start to fall idle at the end
     // of the XCD's queue, so the zero-fill fills the tail of the kernel
     // instead of competing with the k loops for memory bandwidth.
-    const int xcd = blockIdx.x % NUM_XCD, q = blockIdx.x / NUM_XCD;
-    const int ntot = __builtin_amdgcn_readfirstlane(sched[NUM_XCD + xcd]);
+    const int xcd = blockIdx.x % n_xcd, q = blockIdx.x / n_xcd;
+    const int ntot = __builtin_amdgcn_readfirstlane(sched[MAX_XCD + xcd]);
     if (q >= ntot) return;
     const int32_t *seq = order + (int64_t)xcd * P;
     const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
@@ -422,36 +422,36 @@ hipError_t gemm_init() {
 }
 
 template <int B, int NBUF>
-static void launch_one(unsigned grid, const unsigned char *pA, const unsigned char *pB, const GateBuffers &g,
+static void launch_one(unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB, const GateBuffers &g,
                        int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C, hipStream_t s) {
     k_gemm<B, NBUF><<<grid, 256, NBUF * GemmCfg<B>::STAGE_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count, g.order,
-                                                                     g.sched, (int)(grid / NUM_XCD), nbM, nbK, nbN,
+                                                                     g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN,
                                                                      nMacN, M, N, C);
 }
 
 template <int B>
-static void launch_tile(int nbuf, unsigned grid, const unsigned char *pA, const unsigned char *pB,
+static void launch_tile(int nbuf, unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB,
                         const GateBuffers &g, int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C,
                         hipStream_t s) {
-    if (nbuf == 3) launch_one<B, 3>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
-    else if (nbuf == 5) launch_one<B, 5>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
-    else launch_one<B, 4>(grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
+    if (nbuf == 3) launch_one<B, 3>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
+    else if (nbuf == 5) launch_one<B, 5>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
+    else launch_one<B, 4>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
 }
 
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, hipStream_t s) {
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
     (void)nMacM;
-    const int rounds = sched_rounds(tile, nbM, nbN);
-    const unsigned grid = (unsigned)(rounds * NUM_XCD * SUPER_M * SUPER_N);
+    const int rounds = sched_rounds(tile, nbM, nbN, n_xcd);
+    const unsigned grid = (unsigned)(rounds * n_xcd * SUPER_M * SUPER_N);
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
     switch (tile) {
-        case 32: launch_tile<32>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 64: launch_tile<64>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 128: launch_tile<128>(g_nbuf, grid, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 32: launch_tile<32>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 64: launch_tile<64>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 128: launch_tile<128>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

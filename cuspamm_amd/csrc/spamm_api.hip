@@ -59,6 +59,7 @@ struct spamm_ctx : Workspace {
     hipStream_t own_stream = nullptr;
     hipStream_t stream = nullptr;
     int last_hip = 0;
+    int n_xcd = MAX_XCD;        // XCDs the GEMM schedule is built for (from the device's CU count)
 
     Workspace parked;           // the workspace that is not live (see in_static)
     bool in_static = false;     // live workspace = carve-outs of the fixed device array
@@ -207,6 +208,13 @@ int spamm_create(spamm_ctx **out, int device) {
     spamm_ctx *c = new (std::nothrow) spamm_ctx();
     if (!c) return SPAMM_ENOMEM;
     c->device = device;
+    // the schedule groups workgroups by XCD (32 CUs sharing an L2): 256 CUs = 8 XCDs; a partitioned
+    // device shows 128 / 64 / 32 CUs; any other CU count gets one flat sequence
+    c->n_xcd = xcds_for_cu_count(prop.multiProcessorCount);
+    if (const char *env = getenv("SPAMM_NUM_XCD")) {      // developer knob: 1, 2, 4 or 8
+        const int n = atoi(env);
+        if (n == 1 || n == 2 || n == 4 || n == 8) c->n_xcd = n;
+    }
     int rc = set_device(c);
     if (rc == SPAMM_OK && hipStreamCreate(&c->own_stream) != hipSuccess) rc = SPAMM_EHIP;
     c->stream = c->own_stream;
@@ -364,11 +372,11 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->macro_list, (size_t)s.n_macro * s.nbK * sizeof(MacroEntry)))) return rc;
     if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
     if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
-    if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * NUM_XCD * SUPER_M * SUPER_N * 4))) return rc;
-    if ((rc = ensure(c, c->sched, 2 * NUM_XCD * 4))) return rc;
+    if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * MAX_XCD * SUPER_M * SUPER_N * 4))) return rc;
+    if ((rc = ensure(c, c->sched, 2 * MAX_XCD * 4))) return rc;
     if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
-    HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->stream));
+    HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->n_xcd, c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[3], c->stream)); c->ev_gate = true; }
     c->tau = tau;
     c->have_gate = true;
@@ -384,7 +392,7 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
     HIPCHK(c, launch_gemm(c->packedA.p, c->packedB.p, gate_buffers(c), c->M, c->K, c->N, c->tile, dC,
-                          c->stream));
+                          c->n_xcd, c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[4], c->stream)); c->ev_gemm = true; }
     return SPAMM_OK;
 }
@@ -496,8 +504,8 @@ static size_t carve_static(Workspace &w, const spamm_params *p, unsigned char *b
     take(w.macro_list, n_macro * nbK * sizeof(MacroEntry));
     take(w.macro_count, n_macro * 8);
     take(w.macro_work, n_macro * 4);
-    take(w.order, (size_t)sched_rounds(p->tile, (int64_t)nbM, (int64_t)nbN) * NUM_XCD * SUPER_M * SUPER_N * 4);
-    take(w.sched, 2 * NUM_XCD * 4);
+    take(w.order, (size_t)sched_rounds(p->tile, (int64_t)nbM, (int64_t)nbN) * MAX_XCD * SUPER_M * SUPER_N * 4);
+    take(w.sched, 2 * MAX_XCD * 4);
     take(w.kept_total, 16);
     return off;
 }

@@ -29,14 +29,25 @@ inline int macro_dim(int tile) { return 256 / tile; }
 // XCD's L2.
 constexpr int SUPER_M = 4;
 constexpr int SUPER_N = 8;
-constexpr int NUM_XCD = 8;
+constexpr int MAX_XCD = 8;      // an unpartitioned MI355X: 8 XCDs of 32 CUs
 
-// Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin.
-inline int sched_rounds(int tile, int64_t nbM, int64_t nbN) {
+// Number of XCDs the schedule is built for: workgroup b of a grid runs on XCD b % n.  Derived
+// from the CU count of the device (or partition): 32 CUs per XCD; anything that is not 1, 2, 4 or
+// 8 whole XCDs gets one flat sequence (n = 1), which is correct on any device and only gives up
+// the sharing of operand panels in an XCD's L2.
+inline int xcds_for_cu_count(int cus) {
+    for (int n = MAX_XCD; n >= 1; n >>= 1)
+        if (cus == n * SUPER_M * SUPER_N) return n;
+    return 1;
+}
+
+// Workgroups per XCD in the GEMM grid: whole super tiles, dealt round-robin over n_xcd XCDs.
+// (Buffers are sized for n_xcd = MAX_XCD, which is an upper bound for every smaller power of two.)
+inline int sched_rounds(int tile, int64_t nbM, int64_t nbN, int n_xcd = MAX_XCD) {
     const int MT = 256 / tile;
     const int nMacM = (int)((nbM + MT - 1) / MT), nMacN = (int)((nbN + MT - 1) / MT);
     const int n_super = ((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N);
-    return (n_super + NUM_XCD - 1) / NUM_XCD;
+    return (n_super + n_xcd - 1) / n_xcd;
 }
 
 // One entry of a macro tile's union k list: tile column/row k of the
@@ -58,8 +69,8 @@ struct GateBuffers {
     MacroEntry *macro_list; // [n_macro*nbK]   union list of k per macro tile
     int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
     int32_t *macro_work;    // [n_macro]       kept products in the macro tile
-    int32_t *order;         // [8 * P]         macro tile of XCD x's q-th workgroup (P = rounds * 32), valid for q < sched[8 + x]
-    int32_t *sched;         // [16]            per XCD: computing items, all items
+    int32_t *order;         // [n_xcd * P]     macro tile of XCD x's q-th workgroup (P = rounds * 32), valid for q < sched[8 + x]
+    int32_t *sched;         // [16]            per XCD x: [x] computing items, [8 + x] all items
     int64_t *kept_total;    // [1]  kept products
 };
 
@@ -101,7 +112,7 @@ inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
 inline size_t order_lds_limit() { return 64 * 1024; }
 hipError_t gate_init();   // one-time kernel attribute set-up
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
-                       float tau, hipStream_t s);
+                       float tau, int n_xcd, hipStream_t s);
 // per-tile ascending k lists [n_tiles x nbK] from the gate's bitmaps (read-back only)
 hipError_t launch_klist(const uint64_t *mask, uint16_t *klist, int64_t n_tiles, int64_t nbK, hipStream_t s);
 
@@ -127,6 +138,6 @@ hipError_t launch_tau_count(const float *nA, const float *nBt, int64_t nbM, int6
 
 hipError_t gemm_init();   // one-time kernel attribute set-up
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, hipStream_t s);
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, hipStream_t s);
 
 }  // namespace spamm

@@ -15,7 +15,7 @@ TILE = 64
 C_REL_TOL = 1e-3
 
 
-def _full_case(orc, ctx, kind, lam, ratio=None, tau=None, N=N):
+def _full_case(orc, ctx, kind, lam, ratio=None, tau=None, N=N, reachable=True):
     import torch
     sample_rows = [0, (N // TILE) // 3 + 12, N // TILE - 1]
     tab = orc.decay_table(kind, N, lam)
@@ -29,9 +29,15 @@ def _full_case(orc, ctx, kind, lam, ratio=None, tau=None, N=N):
     del A, B
     nA, nB = orc.normmap(hA, TILE, 0), orc.normmap(hB, TILE, 1)
     if tau is None:
+        # a ratio no tau > 0 reaches gives the smallest positive norm product: the largest kept fraction
         tau, ach = orc.tau_for_ratio(nA, nB, ratio)
-        assert abs(ach - ratio) < 0.01
+        assert tau > 0
+        assert (abs(ach - ratio) < 0.01) == reachable
     C = ctx.multiply(dA, dB, TILE, tau)
+    if ratio is not None:
+        # the device's order statistic picks the same threshold from its own norm maps
+        dtau, dach = ctx.tau_for_ratio(ratio)
+        assert np.float32(dtau) == np.float32(tau) and abs(dach - ach) < 1e-12
     del dA, dB
     assert np.array_equal(ctx.get_normmap(0).view(np.uint32), nA.view(np.uint32))
     assert np.array_equal(ctx.get_normmap(1).view(np.uint32), nB.view(np.uint32))
@@ -73,6 +79,25 @@ def test_config2_n8192_ten_percent(orc, ctx):
 
 def test_config3_algebraic_decay_twenty_percent(orc, ctx):
     _full_case(orc, ctx, "alg", 0.0, ratio=0.20)
+
+
+def test_config3_sweep_five_percent(orc, ctx):
+    kept = _full_case(orc, ctx, "alg", 0.0, ratio=0.05)
+    assert abs(kept / 256 ** 3 - 0.05) < 0.01
+
+
+def test_config3_sweep_largest_reachable_fraction(orc, ctx):
+    # the sweep's 50 % point cannot be reached: 1/(1+d)^2 is exactly zero in fp16 beyond d ~ 5790,
+    # so no tau > 0 keeps more than ~36 %; the smallest positive norm product stands in for it
+    kept = _full_case(orc, ctx, "alg", 0.0, ratio=1.0, reachable=False)
+    assert 0.30 < kept / 256 ** 3 < 0.45
+
+
+def test_config2_literal_decay_rate(orc, ctx):
+    # N = 8192 with exp(-0.1 d) as written: at most ~0.3 % of the products are non-zero after fp16
+    # rounding, whatever tau > 0 -- the achieved fraction is reported, not substituted
+    kept = _full_case(orc, ctx, "exp", 0.1, ratio=0.10, N=8192, reachable=False)
+    assert 0 < kept / 128 ** 3 < 0.005
 
 
 def test_config4_dense_tau_zero(orc, ctx):
@@ -125,10 +150,10 @@ def test_power_of_two_scaling_is_exact(orc, ctx):
 N5, TILE5 = 65536, 128
 
 
-def test_config5_n65536_tile128_two_percent(orc, ctx):
+def _config5_case(orc, ctx, lam, reachable):
     import torch
     nb = N5 // TILE5
-    tab = orc.decay_table("exp", N5, 0.003)
+    tab = orc.decay_table("exp", N5, lam)
     dA = torch.empty((N5, N5), dtype=torch.float32, device="cuda")
     dB = torch.empty((N5, N5), dtype=torch.float32, device="cuda")
     ctx.fill_decay(dA, tab, 1)
@@ -136,7 +161,7 @@ def test_config5_n65536_tile128_two_percent(orc, ctx):
     ctx.normmap_f32(1, dB, TILE5)
     ctx.normmap_f32(0, dA, TILE5)
     tau, ach = ctx.tau_for_ratio(0.02)
-    assert abs(ach - 0.02) < 0.002
+    assert tau > 0 and (abs(ach - 0.02) < 0.002) == reachable
     C = ctx.multiply(dA, dB, TILE5, tau)
     nA, nB = ctx.get_normmap(0), ctx.get_normmap(1)
     # Frobenius invariant of the norm maps against the fp16-rounded inputs (row blocks, fp64)
@@ -152,7 +177,7 @@ def test_config5_n65536_tile128_two_percent(orc, ctx):
     assert np.array_equal(ctx.get_counts(), counts)
     st = ctx.get_stats()
     assert st.kept_products == kept and st.total_products == nb ** 3
-    assert abs(kept / nb ** 3 - 0.02) < 0.002
+    assert abs(ach - kept / nb ** 3) < 1e-12
     # C against the exact fp64 product of the resident fp16 operands, on two row slabs
     bound = ctx.dropped_bound(tau)
     for r0 in (0, 30080):
@@ -162,6 +187,17 @@ def test_config5_n65536_tile128_two_percent(orc, ctx):
     zero_rows = C.view(nb, TILE5, nb, TILE5).abs().amax(dim=(1, 3)).cpu().numpy()
     assert np.all(zero_rows[counts == 0] == 0)
     assert np.all(zero_rows[counts > 0] > 0)
+    return kept / nb ** 3
+
+
+def test_config5_n65536_tile128_two_percent(orc, ctx):
+    assert abs(_config5_case(orc, ctx, 0.003, True) - 0.02) < 0.002
+
+
+def test_config5_literal_decay_rate(orc, ctx):
+    # exp(-0.05 d) as written is exactly zero in fp16 beyond d = 346: only a band three tiles wide
+    # is non-zero and at most ~0.02 % of the products can be kept, whatever tau > 0
+    assert 0 < _config5_case(orc, ctx, 0.05, False) < 0.001
 
 
 def test_all_ones_closed_form_n65536(ctx):

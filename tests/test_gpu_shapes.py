@@ -96,3 +96,33 @@ def test_non_finite_inputs_follow_ieee_compare(orc, ctx):
     fin = np.isfinite(Cr)
     assert np.linalg.norm(Cg[fin] - Cr[fin]) <= C_REL_TOL * np.linalg.norm(Cr[fin])
     assert not ref["mask"][0, 0, 0] & np.uint64(2)      # (i=0, j=0, k=1): inf * 0 is not kept
+
+
+@pytest.mark.parametrize("n_xcd", [1, 2, 4])
+def test_schedule_for_other_xcd_counts_gives_the_same_product(orc, ctx, n_xcd, monkeypatch):
+    """The GEMM schedule is built for the device's XCD count (8 on a whole MI355X); a partitioned
+    device, or one that is not whole XCDs of 32 CUs, gets 4 / 2 / 1 sequences.  The schedule only
+    decides where and when a macro tile runs: mask and C must not change by a bit."""
+    import torch
+    import cuspamm_amd as sp
+    monkeypatch.setenv("SPAMM_NUM_XCD", str(n_xcd))          # read once, when the context is created
+    other = sp.SpammContext(0)
+    monkeypatch.delenv("SPAMM_NUM_XCD")
+    try:
+        for (M, K, N), tile, lam, ratio in [((2304, 1024, 4352), 64, 0.004, 0.3), ((1280, 512, 768), 32, 0.01, 0.5),
+                                            ((2048, 2048, 2048), 128, 0.002, 0.2), ((8192, 256, 10240), 64, 0.0, 1.0)]:
+            tab = orc.decay_table("exp", max(M, K, N), lam)
+            A, B = orc.fill_decay(M, K, tab, 1), orc.fill_decay(K, N, tab, 2)
+            dA, dB = _dev(A), _dev(B)
+            ctx.normmap_f32(1, dB, tile)
+            ctx.normmap_f32(0, dA, tile)
+            tau = 0.0 if ratio == 1.0 else ctx.tau_for_ratio(ratio)[0]
+            want = ctx.multiply(dA, dB, tile, tau)
+            mask = ctx.get_mask()
+            got = other.multiply(dA, dB, tile, tau)
+            assert np.array_equal(other.get_mask(), mask)
+            assert torch.equal(got, want)
+        tab = orc.decay_table("exp", 1024, 0.01)
+        _check(orc, other, orc.fill_decay(768, 1024, tab, 3), orc.fill_decay(1024, 640, tab, 4), 64, 0.3)
+    finally:
+        other.close()

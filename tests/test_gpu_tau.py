@@ -65,6 +65,28 @@ def test_reference_bisection(orc, ctx):
             assert abs(ach_g - expected) < 0.01
 
 
+def test_bisection_iterates_match_the_hand_worked_sequence(ctx):
+    # the sequences worked by hand from tool.cu:445-486 (products 1, 2, 3, 4; all sums exact)
+    from test_oracle_gate import BISECT_HAND
+    ctx.set_normmaps(np.array([[1.0, 2.0, 3.0, 4.0]], dtype=np.float32), np.ones((4, 1), dtype=np.float32), 32)
+    for expected, seq in BISECT_HAND.items():
+        for rounds, want in enumerate(seq, start=1):
+            assert ctx.tune_bisect(expected, 0.01, rounds) == want, (expected, rounds)
+    assert ctx.tune_bisect(0.25, 0.01, 20) == (3.75, 0.25)
+    assert ctx.tune_bisect(0.75, 0.01, 20) == (1.25, 0.75)
+
+
+def test_dropped_bound_hand_worked(ctx):
+    # per output tile the dropped products sum to 7, 10, 4, 8 at tau = 10 and to 7, 2, 4, 0 at
+    # tau = 8 (a product equal to tau is kept)
+    nA = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)
+    nB = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    ctx.set_normmaps(nA, nB, 32)
+    assert ctx.dropped_bound(10.0) == pytest.approx(np.sqrt(229.0), rel=1e-14)
+    assert ctx.dropped_bound(8.0) == pytest.approx(np.sqrt(69.0), rel=1e-14)
+    assert ctx.dropped_bound(0.0) == 0.0
+
+
 def test_full_size_selection(orc, ctx):
     import torch
     N, tile = 16384, 64

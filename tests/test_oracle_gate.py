@@ -109,6 +109,37 @@ def test_tau_for_ratio_and_bisection(orc):
     assert abs(orc.gate(nA, nB, tau)[0] / (8 * 32 * 8) - ach) < 1e-6
 
 
+# tuneValidRate worked by hand from tool.cu:445-486 on the 1 x 4 x 1 map with products 1, 2, 3, 4
+# (kept ratio is a multiple of 1/4, so targets 0.6 and 0.1 are never met and the loop runs until
+# max_rounds).  Round 0 measures the ratio at Norm = 0 (1.0) and moves to the mean product 2.5 = up.
+#   expected 0.6: 2.5 (ratio .5 < .6: up = 2.5, Norm = (2.5 + 0) / 2)  -> 1.25 (.75 > .6: down = 1.25,
+#     Norm = (1.25 + 2.5) / 2) -> 1.875 (.75: down = 1.875) -> 2.1875 (.5: up = 2.1875) -> 2.03125
+#     (.5: up) -> 1.953125 (.75: down) -> 1.9921875
+#   expected 0.1: 2.5 (.5 > .1 and up == Norm: up = 5, down = 2.5) -> 3.75 (.25 > .1: down = 3.75)
+#     -> 4.375 (0 < .1: up = 4.375) -> 4.0625 (0: up) -> 3.90625 (.25: down) -> 3.984375
+# The value returned after r rounds is the Norm entering round r; the ratio is the one measured in
+# round r - 1.
+BISECT_HAND = {
+    0.6: [(2.5, 1.0), (1.25, 0.5), (1.875, 0.75), (2.1875, 0.75), (2.03125, 0.5), (1.953125, 0.5), (1.9921875, 0.75)],
+    0.1: [(2.5, 1.0), (3.75, 0.5), (4.375, 0.25), (4.0625, 0.0), (3.90625, 0.0), (3.984375, 0.25)],
+}
+
+
+def test_bisection_iterates_match_the_hand_worked_sequence(orc):
+    nA = np.array([[1.0, 2.0, 3.0, 4.0]], dtype=np.float32)
+    nB = np.ones((4, 1), dtype=np.float32)
+    for expected, seq in BISECT_HAND.items():
+        for rounds, (norm, rate) in enumerate(seq, start=1):
+            tau, ach = orc.tune_bisect(nA, nB, expected, 0.01, rounds)
+            assert (tau, ach) == (norm, rate), (expected, rounds, tau, ach)
+    # targets that are met stop early: 0.5 after round 1 (Norm 2.5 keeps 3 and 4), 0.25 after the
+    # doubling step (3.75 keeps 4), 0.75 after one halving (1.25 keeps 2, 3, 4), 1.0 at once (Norm 0)
+    assert orc.tune_bisect(nA, nB, 0.5, 0.01, 20) == (2.5, 0.5)
+    assert orc.tune_bisect(nA, nB, 0.25, 0.01, 20) == (3.75, 0.25)
+    assert orc.tune_bisect(nA, nB, 0.75, 0.01, 20) == (1.25, 0.75)
+    assert orc.tune_bisect(nA, nB, 1.0, 0.01, 20) == (0.0, 1.0)
+
+
 def test_zero_tail_gives_smallest_positive_tau(orc):
     nA = np.array([[1.0, 0.0, 0.0, 0.0]], dtype=np.float32)
     nB = np.ones((4, 1), dtype=np.float32)

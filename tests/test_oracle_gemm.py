@@ -104,6 +104,25 @@ def test_dropped_norm_bound(orc):
     assert 0 < r["kept"] < nb ** 3
 
 
+def test_dropped_bound_hand_worked(orc):
+    # nA = [[1,2,3],[4,5,6]], nB = [[1,2],[3,4],[5,6]]; products per output tile (k = 0,1,2):
+    #   (0,0): 1, 6, 15   (0,1): 2, 8, 18   (1,0): 4, 15, 30   (1,1): 8, 20, 36
+    # tau = 10 drops everything below 10: sums 7, 10, 4, 8 -> sqrt(49 + 100 + 16 + 64) = sqrt(229)
+    # tau = 8 keeps the two products equal to 8 (>=): sums 7, 2, 4, 0 -> sqrt(69)
+    nA = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)
+    nB = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    assert orc.dropped_bound(nA, nB, 10.0) == pytest.approx(np.sqrt(229.0), rel=1e-15)
+    assert orc.dropped_bound(nA, nB, 8.0) == pytest.approx(np.sqrt(69.0), rel=1e-15)
+    assert orc.dropped_bound(nA, nB, 10.0, 1, 2) == pytest.approx(np.sqrt(80.0), rel=1e-15)      # tile row 1 only
+    assert orc.dropped_bound(nA, nB, 0.0) == 0.0                                                  # nothing dropped
+    assert orc.dropped_bound(nA, nB, 37.0) == pytest.approx(np.sqrt(22.0 ** 2 + 28.0 ** 2 + 49.0 ** 2 + 64.0 ** 2), rel=1e-15)
+    # the product that is compared is the fp32 one: 3 * (1/3 rounded) is exactly 1 in fp32, so it is
+    # kept at tau = 1 although the exact product of the two floats lies just above or below 1
+    third = np.float32(1.0) / np.float32(3.0)
+    assert np.float32(3.0) * third == np.float32(1.0)
+    assert orc.dropped_bound(np.array([[3.0]], dtype=np.float32), np.array([[third]], dtype=np.float32), 1.0) == 0.0
+
+
 def test_row_slab_interface(orc):
     b, n = 32, 128
     A, B = _inputs(orc, n, n, n, 0.02)
