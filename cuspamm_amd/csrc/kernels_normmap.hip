@@ -39,8 +39,12 @@ __device__ __forceinline__ float butterfly64(float v) {
     return v;
 }
 
-// One workgroup (4 waves) per strip of B rows x SW columns (SW/B tiles; SW =
-// 256, or 128 for B = 128 so that the strip still fits 3 workgroups per CU).
+// One workgroup (4 waves) per strip of B rows x SW columns (SW/B tiles, SW =
+// 256: every row segment a wave reads is 1 KiB).  The tiles of a strip pass
+// through LDS in PH phases of SW/B/PH tiles each (PH = 2 for B = 128: one
+// 32 KiB tile at a time, so that three workgroups still fit a CU while their
+// loads -- all issued before the first phase -- cover the whole 256-column strip;
+// 512-byte row segments cost 4-9 % of the bandwidth).
 //   load    every wave-wide load covers 64*4/SW full strip rows, each SW*4
 //           contiguous bytes; a lane takes whole 8-row groups; all loads of a
 //           lane are in flight together.
@@ -54,34 +58,46 @@ __device__ __forceinline__ float butterfly64(float v) {
 //   store   after one barrier: the tiles are copied out with contiguous 1 KiB
 //           wave stores (a packed tile is one contiguous block in memory), and
 //           one wave per tile applies the canonical reduction.
-template <int B, int ROLE, int SW, bool IN16>
-__global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
+// (The phased A role is held to three waves per SIMD: it gains more from a third resident
+// workgroup than it loses to a few spilled registers; the B role would spill far more.)
+template <int B, int ROLE, int SW, bool IN16, int PH = 1>
+__global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT, uint4 *__restrict__ packed2,
                                                  float *__restrict__ nm2, const float *__restrict__ rowmax,
                                                  float tau_skip) {
     constexpr int TPS = SW / B;           // tiles per strip
-    constexpr int LPR = SW / 4;           // lanes across one strip row
-    constexpr int RH = 64 / LPR;          // strip rows per wave-wide load
+    constexpr int TPP = TPS / PH;         // tiles per phase (resident in LDS together)
+    static_assert(TPP * PH == TPS && TPP >= 1, "phases must divide the strip's tiles");
+    // Lane -> element mapping.  PH = 1: a wave-wide load covers whole strip rows (LPR lanes
+    // each).  PH > 1: the waves are split between the phases' tiles (WPP waves per phase), a
+    // wave-wide load covers rows of its own tiles only (the waves of the other phases read the
+    // neighbouring segments of the same rows at the same time), and a phase is staged by whole
+    // waves.
+    constexpr int WPP = 4 / PH;                        // waves per phase
+    constexpr int LPR = (PH > 1 ? TPP * B : SW) / 4;   // lanes across one row of the wave's columns
+    constexpr int RH = 64 / LPR;                       // rows per wave-wide load
+    constexpr int GSTEP = WPP * RH;                    // 8-row groups between a lane's groups
+    static_assert(PH == 1 || PH == 2 || PH == 4, "phases are made of whole waves");
     constexpr int QN = B / 8;             // k-groups per tile
     constexpr int VPT = B * B / 8;        // 16-byte vectors per tile
     constexpr int QS = B * 16 + 16;       // bytes per k-group segment in LDS (padded)
     constexpr int TS = QN * QS;           // bytes per tile in LDS
     constexpr int PITCH = QN + 1;         // padded row of the chunk-sum table
     constexpr int CH = B * PITCH;         // floats per tile in the chunk-sum table
-    constexpr int NGW = B / (32 * RH);    // 8-row groups per lane
+    constexpr int NGW = B / (8 * GSTEP);  // 8-row groups per lane
     constexpr int STEPS = VPT / 64;
-    __shared__ __attribute__((aligned(16))) unsigned char s_pack[TPS * TS];
-    __shared__ float s_chunk[TPS * CH];
+    __shared__ __attribute__((aligned(16))) unsigned char s_pack[TPP * TS];
+    __shared__ float s_chunk[TPP * CH];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int64_t I = blockIdx.x / nstrip;            // tile row of the strip
     const int64_t sc = blockIdx.x % nstrip;
     const int64_t col0 = sc * SW;
-    const int cl = 4 * (lane % LPR);                  // first column of this lane inside the strip
-    const int g0 = wave * RH + lane / LPR;            // first 8-row group of this lane; then every 4*RH-th
+    const int cl = (wave / WPP) * (TPP * B) + 4 * (lane % LPR);   // first column of this lane inside the strip
+    const int g0 = (wave % WPP) * RH + lane / LPR;    // first 8-row group of this lane; then every GSTEP-th
     const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
     const bool valid = col0 + cl < cols;
     // IN16: the input already is fp16 (the reference's own input type, para.h:1); the
@@ -93,7 +109,7 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
     for (int i = 0; i < NGW; i++)
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const int r = 8 * (g0 + 4 * RH * i) + j;
+            const int r = 8 * (g0 + GSTEP * i) + j;
             if (!valid) {
                 v[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             } else if (IN16) {
@@ -109,13 +125,15 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
 
     // ROLE 2 = the same matrix is both operands (A = B): one read of X, both packed layouts and
     // both norm maps (A role first -> packed/nm, then B role -> packed2/nm2/nmT), LDS reused.
-    auto stage_a = [&]() {
+    auto stage_a = [&](int ph) {
         const int q = cin / 8, h = (cin % 8) / 4;
+        if (PH > 1 && t / TPP != ph) return;
+        const int t = (cl / B) % TPP;      // tile inside the phase
 #pragma unroll
         for (int i = 0; i < NGW; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const int r = 8 * (g0 + 4 * RH * i) + j;
+                const int r = 8 * (g0 + GSTEP * i) + j;
                 const _Float16 h0 = (_Float16)v[i][j].x, h1 = (_Float16)v[i][j].y;
                 const _Float16 h2 = (_Float16)v[i][j].z, h3 = (_Float16)v[i][j].w;
                 const float f0 = (float)h0, f1 = (float)h1, f2 = (float)h2, f3 = (float)h3;
@@ -134,10 +152,12 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
                 if (h) s_chunk[t * CH + r * PITCH + q] = s8;
             }
     };
-    auto stage_b = [&]() {
+    auto stage_b = [&](int ph) {
+        if (PH > 1 && t / TPP != ph) return;
+        const int t = (cl / B) % TPP;      // tile inside the phase
 #pragma unroll
         for (int i = 0; i < NGW; i++) {
-            const int kg = g0 + 4 * RH * i;
+            const int kg = g0 + GSTEP * i;
             uint4 o[4];
             float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             o[0].x = cvt_pack2(v[i][0].x, v[i][1].x, s[0]);
@@ -164,13 +184,13 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
         }
     };
     // packed tiles out (256 threads x 16 bytes = 4 KiB per step, contiguous per tile)
-    __shared__ int s_skip[TPS];
-    auto copy_out = [&](bool as_b, uint4 *__restrict__ pk, bool prune) {
+    __shared__ int s_skip[TPP];
+    auto copy_out = [&](int ph, bool as_b, uint4 *__restrict__ pk, bool prune) {
 #pragma unroll
-        for (int i = 0; i < TPS * VPT / 256; i++) {
+        for (int i = 0; i < TPP * VPT / 256; i++) {
             const int vi = threadIdx.x + 256 * i;
             const int tt = vi / VPT, iv = vi % VPT;
-            const int64_t Jt = sc * TPS + tt;
+            const int64_t Jt = sc * TPS + ph * TPP + tt;
             if (Jt < nbc && !(prune && s_skip[tt])) {
                 const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
                 const int64_t tile = as_b ? Jt * nbr + I : I * nbc + Jt;
@@ -184,9 +204,9 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
     // bound is below tau is never read by the GEMM and its fp16 copy need not be written.  The
     // bound is max_j nB[k,j] for the A pass (B's norm map is complete by then) and the largest
     // finite float for the B pass, which runs first: there only tiles of norm zero are left out.
-    auto norms = [&](bool as_b, float *__restrict__ nmo, float *__restrict__ nmTo, bool prune) {
-        for (int tt = wave; tt < TPS; tt += 4) {
-            const int64_t Jt = sc * TPS + tt;
+    auto norms = [&](int ph, bool as_b, float *__restrict__ nmo, float *__restrict__ nmTo, bool prune) {
+        for (int tt = wave; tt < TPP; tt += 4) {
+            const int64_t Jt = sc * TPS + ph * TPP + tt;
             if (Jt >= nbc) break;
             const float rmax = prune ? (rowmax != nullptr ? rowmax[Jt] : 3.402823466e+38f) : 0.0f;
             float partial = 0.0f;
@@ -204,52 +224,34 @@ __global__ __launch_bounds__(256) void k_normmap(const void *__restrict__ Xv, in
             }
         }
     };
-    auto emit = [&](bool as_b, uint4 *__restrict__ pk, float *__restrict__ nmo, float *__restrict__ nmTo) {
-        copy_out(as_b, pk, false);
-        norms(as_b, nmo, nmTo, false);
+    // one operand role: the strip's tiles go through LDS phase by phase
+    auto emit_role = [&](bool as_b, uint4 *__restrict__ pk, float *__restrict__ nmo, float *__restrict__ nmTo,
+                         bool prune) {
+#pragma unroll
+        for (int ph = 0; ph < PH; ph++) {
+            if (ph) __syncthreads();           // the previous phase's tiles have been copied out
+            if (as_b) stage_b(ph); else stage_a(ph);
+            __syncthreads();
+            if (prune) {
+                norms(ph, as_b, nmo, nmTo, true);
+                __syncthreads();
+                copy_out(ph, as_b, pk, true);
+            } else {
+                copy_out(ph, as_b, pk, false);
+                norms(ph, as_b, nmo, nmTo, false);
+            }
+        }
     };
+    const bool prune = tau_skip > 0.0f;
     if (ROLE == 0) {
-        stage_a();
-        __syncthreads();
-        if (tau_skip > 0.0f) {
-            norms(false, nm, nullptr, true);
-            __syncthreads();
-            copy_out(false, packed, true);
-        } else {
-            emit(false, packed, nm, nullptr);
-        }
+        emit_role(false, packed, nm, nullptr, prune);
     } else if (ROLE == 1) {
-        stage_b();
-        __syncthreads();
-        if (tau_skip > 0.0f) {
-            norms(true, nm, nmT, true);
-            __syncthreads();
-            copy_out(true, packed, true);
-        } else {
-            emit(true, packed, nm, nmT);
-        }
+        emit_role(true, packed, nm, nmT, prune);
     } else {
         // one pass for both roles: no row maxima yet, so only tiles of norm zero are left out
-        const bool prune = tau_skip > 0.0f;
-        stage_a();
+        emit_role(false, packed, nm, nullptr, prune);
         __syncthreads();
-        if (prune) {
-            norms(false, nm, nullptr, true);
-            __syncthreads();
-            copy_out(false, packed, true);
-        } else {
-            emit(false, packed, nm, nullptr);
-        }
-        __syncthreads();
-        stage_b();
-        __syncthreads();
-        if (prune) {
-            norms(true, nm2, nmT, true);
-            __syncthreads();
-            copy_out(true, packed2, true);
-        } else {
-            emit(true, packed2, nm2, nmT);
-        }
+        emit_role(true, packed2, nm2, nmT, prune);
     }
 }
 
@@ -341,13 +343,13 @@ static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int 
                                  float *nmT, hipStream_t s, void *packed2 = nullptr, float *nm2 = nullptr,
                                  const float *rowmax = nullptr, float tau_skip = 0.0f) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
-    const int sw = tile == 128 ? 128 : 256;
+    const int sw = 256;
     const int64_t nstrip = (cols + sw - 1) / sw;
     const unsigned grid = (unsigned)(nbr * nstrip);
     switch (tile) {
         case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
-        case 128: k_normmap<128, ROLE, 128, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 128: k_normmap<128, ROLE, 256, IN16, 2><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
