@@ -283,10 +283,17 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // round-robin over the n_xcd XCDs of the device, so workgroup b runs on XCD
 // b % n_xcd and is the (b / n_xcd)-th workgroup that XCD starts (n_xcd = 1: one
 // flat sequence, for devices that are not whole XCDs of 32 CUs).
-//   1. Super tiles are ranked by descending kept-product count and dealt to
-//      the XCDs in snake order: every XCD owns whole super tiles, so the
-//      workgroups sharing one L2 share A row panels and B column panels, and
-//      the XCDs get equal work.
+//   1. Super tiles are ranked by descending length (entries of their macro
+//      tiles' union lists: that, not the kept-product count, is the time a
+//      workgroup takes) and dealt to the XCDs: every XCD owns whole super
+//      tiles, so the workgroups sharing one L2 share A row panels and B column
+//      panels.  Up to LPT_MAX_SUPER super tiles are dealt greedily, each to the
+//      XCD with the least length so far (at most `rounds` per XCD, the size
+//      the grid and the order buffer are laid out for); a plain snake deal by
+//      rank leaves XCDs up to 18 % apart when a problem has only a few super
+//      tiles per XCD, and the slowest XCD sets the kernel's time.  Beyond that
+//      size the deal is the snake (the serial greedy loop would take longer
+//      than it saves, and many super tiles per XCD even out by themselves).
 //   2. Inside an XCD the computing macro tiles run super tile by super tile
 //      (measured on banded inputs, heaviest-first classes inside an XCD did
 //      not shorten the tail but pulled neighbours apart: 10 % more L2 misses).
@@ -298,11 +305,13 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
                                                 int n_super, int rounds, int n_xcd) {
-    extern __shared__ int swork[];               // [n_super] work, then [n_super] super tile origin by rank
-    int *srank_id = swork + n_super;
+    extern __shared__ int swork[];               // [n_super] length, then [n_super] super tile origin by rank,
+    int *srank_id = swork + n_super;             // then (greedy deal only) [n_xcd][rounds] rank of each XCD's r-th super tile
+    uint16_t *sdeal = reinterpret_cast<uint16_t *>(srank_id + n_super);
     __shared__ unsigned long long total;
+    __shared__ int s_nonempty;
     const int P = rounds * SUPER_M * SUPER_N;
-    if (threadIdx.x == 0) total = 0;
+    if (threadIdx.x == 0) { total = 0; s_nonempty = 0; }
     // (this kernel is one workgroup on an idle GPU: its run time is memory round trips and
     // instruction fetch, so every thread takes one macro tile row of one super tile -- all loads
     // of the kernel's first step are in flight at once -- and the code is kept small)
@@ -312,11 +321,14 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     for (int e = threadIdx.x; e < n_super * SUPER_M; e += blockDim.x) {
         const int sid = e / SUPER_M, a = e % SUPER_M;
         const int mi = (sid / nSupN) * SUPER_M + a, mj0 = (sid % nSupN) * SUPER_N;
-        int w = 0;
+        int w = 0, len = 0;
 #pragma unroll
         for (int b = 0; b < SUPER_N; b++)
-            if (mi < nMacM && mj0 + b < nMacN) w += g.macro_work[mi * nMacN + mj0 + b];
-        if (w) atomicAdd(&swork[sid], w);
+            if (mi < nMacM && mj0 + b < nMacN) {
+                w += g.macro_work[mi * nMacN + mj0 + b];
+                len += g.macro_count[2 * (mi * nMacN + mj0 + b)];
+            }
+        if (len) atomicAdd(&swork[sid], len);
         mine += (unsigned long long)w;
     }
     if (mine) atomicAdd(&total, mine);
@@ -329,14 +341,66 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
             rank += (wj > w) || (wj == w && j < sid);
         }
         srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
+        if (n_super <= LPT_MAX_SUPER) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
+        if (w > 0) atomicAdd(&s_nonempty, 1);
     }
     __syncthreads();
+    // the serial part of the greedy deal costs ~0.2 us per super tile with work: worth it only
+    // while there are few of them (that is also where the snake leaves the XCDs furthest apart)
+    const int n_ne = s_nonempty;
+    const bool greedy = n_super <= LPT_MAX_SUPER && n_ne <= LPT_GREEDY_MAX;
+    if (greedy) {
+        // lengths by rank, then the deal
+        int mylen[(LPT_MAX_SUPER + 1023) / 1024], myrank[(LPT_MAX_SUPER + 1023) / 1024];
+        int n = 0;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) { mylen[n] = swork[sid]; myrank[n] = sdeal[sid]; n++; }
+        __syncthreads();
+        n = 0;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) { swork[myrank[n]] = mylen[n]; n++; }
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            // lane x < n_xcd keeps XCD x's length so far and its number of super tiles; the
+            // least-loaded XCD with room is the minimum of (length, lane) over the lanes
+            // (lengths stay far below 2^28: at most LPT_GREEDY_MAX super tiles of 32 lists)
+            const int x = threadIdx.x;
+            uint32_t load = 0;
+            int cnt = 0;
+            for (int r = 0; r < n_ne; r++) {
+                uint32_t key = (x < n_xcd && cnt < rounds) ? (load << 3) | (uint32_t)x : ~0u;
+#pragma unroll
+                for (int off = 1; off < MAX_XCD; off <<= 1) {
+                    const uint32_t o = (uint32_t)__shfl_xor((int)key, off, 64);
+                    key = o < key ? o : key;
+                }
+                if ((int)(key & 7u) == x) {
+                    sdeal[x * rounds + cnt] = (uint16_t)r;
+                    cnt++;
+                    load += (uint32_t)swork[r];
+                }
+            }
+            // super tiles with nothing kept (ranks n_ne ..) fill the XCDs' remaining slots in lane order
+            const int room = x < n_xcd ? rounds - cnt : 0;
+            int before = room;
+#pragma unroll
+            for (int off = 1; off < MAX_XCD; off <<= 1) {
+                const int o = __shfl_up(before, off, 64);
+                if (x >= off) before += o;
+            }
+            before -= room;
+            for (int c = 0; c < room; c++) {
+                const int r = n_ne + before + c;
+                sdeal[x * rounds + cnt + c] = r < n_super ? (uint16_t)r : (uint16_t)0xffffu;   // 0xffff: no super tile
+            }
+        }
+        __syncthreads();
+    }
 
     // macro tile of XCD x at raw position p (round-major, then slot inside the super tile), or -1
     auto macro_at = [&](int x, int p) -> int {
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
-        const int sr = round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
-        if (p >= P || sr >= n_super) return -1;
+        if (p >= P) return -1;
+        const int sr = greedy ? (int)sdeal[x * rounds + round] : round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
+        if (sr >= n_super) return -1;
         const int origin = srank_id[sr];
         const int mi = (origin >> 16) + slot / SUPER_N, mj = (origin & 0xffff) + slot % SUPER_N;
         return (mi < nMacM && mj < nMacN) ? mi * nMacN + mj : -1;
@@ -433,7 +497,7 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;
     const int n_super = nSupM * nSupN;
     const int rounds = (n_super + n_xcd - 1) / n_xcd;
-    k_order<<<1, 1024, (size_t)n_super * 2 * sizeof(int), s>>>(g, nMacM, nMacN, nSupN, n_super, rounds, n_xcd);
+    k_order<<<1, 1024, order_lds_bytes(tile, nbM, nbN), s>>>(g, nMacM, nMacN, nSupN, n_super, rounds, n_xcd);
     return hipGetLastError();
 }
 

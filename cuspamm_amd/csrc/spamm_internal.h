@@ -104,10 +104,15 @@ hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *
 size_t gate_lds_bytes(int tile, int64_t nbK);
 inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k_gate (a few static bytes aside)
 // k_order ranks the super tiles of C (4 x 8 macro tiles of 256 x 256) in one workgroup's LDS
+constexpr int LPT_MAX_SUPER = 2048;     // the greedy deal's table is laid out for at most this many super tiles,
+constexpr int LPT_GREEDY_MAX = 64;      // and it runs while at most this many of them hold any work
 inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
     const int MT = 256 / tile;
     const int64_t nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
-    return (size_t)(((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N)) * 2 * sizeof(int);
+    const size_t n_super = (size_t)(((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N));
+    // length + origin by rank, and for the greedy deal a table of at most MAX_XCD x rounds (or
+    // n_super parked ranks) 16-bit entries
+    return n_super * 2 * sizeof(int) + (n_super <= (size_t)LPT_MAX_SUPER ? (n_super + 2 * MAX_XCD) * sizeof(uint16_t) * 2 : 0);
 }
 inline size_t order_lds_limit() { return 64 * 1024; }
 hipError_t gate_init();   // one-time kernel attribute set-up
