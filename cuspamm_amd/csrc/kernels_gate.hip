@@ -333,24 +333,48 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     }
     if (mine) atomicAdd(&total, mine);
     __syncthreads();
+    // How the super tiles are dealt to the XCDs (sdeal, or the snake formula in macro_at):
+    //   DEAL_LPT    few super tiles hold work: ranked by length, each goes to the XCD with the
+    //               least length so far (pure balance; ~0.2 us of serial work per super tile);
+    //   DEAL_BAND   at most 60 % of the super tiles hold work (a narrow band): ranked in
+    //               row-major order, those with work first; every group of n_xcd consecutive
+    //               ones -- neighbours along the band that read the same operand panels -- runs
+    //               at the same time, one per XCD, and inside a group the heaviest goes to the
+    //               XCD with the least length so far.  Measured against the snake: -4 to -6 %
+    //               GEMM time on exponential-decay bands that keep 10 % (N = 16384), -2 % at
+    //               N = 32768, but +1 to +3 % when most super tiles hold work (algebraic decay,
+    //               30 % kept), hence the condition;
+    //   DEAL_SNAKE  ranked by length, dealt in snake order (no table: any number of super tiles).
+    enum { DEAL_LPT, DEAL_BAND, DEAL_SNAKE };
+    {
+        int ne = 0;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) ne += swork[sid] > 0;
+        if (ne) atomicAdd(&s_nonempty, ne);
+    }
+    __syncthreads();
+    const int n_ne = s_nonempty;
+    const int deal = n_super > LPT_MAX_SUPER ? DEAL_SNAKE
+                     : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT : (5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int w = swork[sid];
         int rank = 0;
-        for (int j = 0; j < n_super; j++) {
-            const int wj = swork[j];
-            rank += (wj > w) || (wj == w && j < sid);
+        if (deal == DEAL_BAND) {
+            for (int j = 0; j < n_super; j++) {
+                const int wj = swork[j];
+                rank += ((wj > 0) > (w > 0)) || ((wj > 0) == (w > 0) && j < sid);
+            }
+        } else {
+            for (int j = 0; j < n_super; j++) {
+                const int wj = swork[j];
+                rank += (wj > w) || (wj == w && j < sid);
+            }
         }
         srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
-        if (n_super <= LPT_MAX_SUPER) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
-        if (w > 0) atomicAdd(&s_nonempty, 1);
+        if (deal != DEAL_SNAKE) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
     }
     __syncthreads();
-    // the serial part of the greedy deal costs ~0.2 us per super tile with work: worth it only
-    // while there are few of them (that is also where the snake leaves the XCDs furthest apart)
-    const int n_ne = s_nonempty;
-    const bool greedy = n_super <= LPT_MAX_SUPER && n_ne <= LPT_GREEDY_MAX;
-    if (greedy) {
-        // lengths by rank, then the deal
+    if (deal != DEAL_SNAKE) {
+        // lengths by rank, then the deal by one wave
         int mylen[(LPT_MAX_SUPER + 1023) / 1024], myrank[(LPT_MAX_SUPER + 1023) / 1024];
         int n = 0;
         for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) { mylen[n] = swork[sid]; myrank[n] = sdeal[sid]; n++; }
@@ -358,7 +382,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         n = 0;
         for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) { swork[myrank[n]] = mylen[n]; n++; }
         __syncthreads();
-        if (threadIdx.x < 64) {
+        if (threadIdx.x < 64 && deal == DEAL_LPT) {
             // lane x < n_xcd keeps XCD x's length so far and its number of super tiles; the
             // least-loaded XCD with room is the minimum of (length, lane) over the lanes
             // (lengths stay far below 2^28: at most LPT_GREEDY_MAX super tiles of 32 lists)
@@ -392,6 +416,47 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
                 sdeal[x * rounds + cnt + c] = r < n_super ? (uint16_t)r : (uint16_t)0xffffu;   // 0xffff: no super tile
             }
         }
+        if (threadIdx.x < 64 && deal == DEAL_BAND) {
+            // lane i holds the i-th super tile of the group, lane x the length of XCD x so far
+            const int x = threadIdx.x;
+            int load = 0, cnt = 0;
+            const int ngroups = (n_ne + n_xcd - 1) / n_xcd;
+            for (int g2 = 0; g2 < ngroups; g2++) {
+                const int r = g2 * n_xcd + x;
+                const int w = (x < n_xcd && r < n_ne) ? swork[r] : -1;           // -1: no super tile
+                int irank = 0, xrank = 0;       // my super tile among the group's, heaviest first; my XCD, shortest first
+#pragma unroll
+                for (int j = 0; j < MAX_XCD; j++) {
+                    const int wj = __builtin_amdgcn_readlane(w, j), lj = __builtin_amdgcn_readlane(load, j);
+                    irank += (wj > w) || (wj == w && j < x);
+                    xrank += (j < n_xcd) && ((lj < load) || (lj == load && j < x));
+                }
+                int mine = -1, wm = -1;         // the super tile whose rank is my XCD's rank
+#pragma unroll
+                for (int j = 0; j < MAX_XCD; j++) {
+                    const int rj = __builtin_amdgcn_readlane(irank, j), wj = __builtin_amdgcn_readlane(w, j);
+                    if (rj == xrank && j < n_xcd) { mine = j; wm = wj; }
+                }
+                if (x < n_xcd && wm > 0) {          // (the last group may have fewer super tiles than XCDs)
+                    sdeal[x * rounds + cnt] = (uint16_t)(g2 * n_xcd + mine);
+                    cnt++;
+                    load += wm;
+                }
+            }
+            // super tiles with nothing kept (ranks n_ne ..) fill the XCDs' remaining slots in lane order
+            const int room = x < n_xcd ? rounds - cnt : 0;
+            int before = room;
+#pragma unroll
+            for (int off = 1; off < MAX_XCD; off <<= 1) {
+                const int o = __shfl_up(before, off, 64);
+                if (x >= off) before += o;
+            }
+            before -= room;
+            for (int c = 0; c < room; c++) {
+                const int r = n_ne + before + c;
+                sdeal[x * rounds + cnt + c] = r < n_super ? (uint16_t)r : (uint16_t)0xffffu;   // 0xffff: no super tile
+            }
+        }
         __syncthreads();
     }
 
@@ -399,7 +464,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     auto macro_at = [&](int x, int p) -> int {
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
         if (p >= P) return -1;
-        const int sr = greedy ? (int)sdeal[x * rounds + round] : round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
+        const int sr = deal != DEAL_SNAKE ? (int)sdeal[x * rounds + round] : round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
         if (sr >= n_super) return -1;
         const int origin = srank_id[sr];
         const int mi = (origin >> 16) + slot / SUPER_N, mj = (origin & 0xffff) + slot % SUPER_N;

@@ -33,7 +33,10 @@ def _full_case(orc, ctx, kind, lam, ratio=None, tau=None, N=N, reachable=True):
         tau, ach = orc.tau_for_ratio(nA, nB, ratio)
         assert tau > 0
         assert (abs(ach - ratio) < 0.01) == reachable
-    C = ctx.multiply(dA, dB, TILE, tau)
+    # every element of C must be written, whatever the schedule: start from NaNs
+    C = torch.full((N, N), float("nan"), dtype=torch.float32, device="cuda")
+    ctx.multiply(dA, dB, TILE, tau, C=C)
+    assert not bool(torch.isnan(C).any())
     if ratio is not None:
         # the device's order statistic picks the same threshold from its own norm maps
         dtau, dach = ctx.tau_for_ratio(ratio)
