@@ -336,7 +336,9 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     // How the super tiles are dealt to the XCDs (sdeal, or the snake formula in macro_at):
     //   DEAL_LPT    few super tiles hold work: ranked by length, each goes to the XCD with the
     //               least length so far (pure balance; ~0.2 us of serial work per super tile);
-    //   DEAL_BAND   at most 60 % of the super tiles hold work (a narrow band): ranked in
+    //   DEAL_BAND   at most BAND_DEAL_MAX super tiles hold work (the deal is serial, ~1.2 us
+    //               per group; at N = 65536 it cost more than it gained) and they are at most
+    //               60 % of all (a narrow band): ranked in
     //               row-major order, those with work first; every group of n_xcd consecutive
     //               ones -- neighbours along the band that read the same operand panels -- runs
     //               at the same time, one per XCD, and inside a group the heaviest goes to the
@@ -354,7 +356,8 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     __syncthreads();
     const int n_ne = s_nonempty;
     const int deal = n_super > LPT_MAX_SUPER ? DEAL_SNAKE
-                     : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT : (5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
+                     : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT
+                        : (n_ne <= BAND_DEAL_MAX && 5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
     for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
         const int w = swork[sid];
         int rank = 0;

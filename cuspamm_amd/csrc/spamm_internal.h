@@ -106,6 +106,7 @@ inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k
 // k_order ranks the super tiles of C (4 x 8 macro tiles of 256 x 256) in one workgroup's LDS
 constexpr int LPT_MAX_SUPER = 2048;     // the greedy deal's table is laid out for at most this many super tiles,
 constexpr int LPT_GREEDY_MAX = 64;      // and it runs while at most this many of them hold any work
+constexpr int BAND_DEAL_MAX = 256;      // the grouped row-major deal runs up to this many super tiles with work
 inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
     const int MT = 256 / tile;
     const int64_t nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
