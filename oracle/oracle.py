@@ -45,6 +45,8 @@ def lib():
     L.orc_fill_decay.argtypes = [_f32p, _i64, _i64, _f32p, ctypes.c_uint64, ctypes.c_int]
     L.orc_normmap.argtypes = [_u16p, _i64, _i64, ctypes.c_int, ctypes.c_int, _f32p]
     L.orc_normmap.restype = ctypes.c_int
+    L.orc_normmap_ref16_model.argtypes = [_u16p, _i64, _i64, _f32p]
+    L.orc_normmap_ref16_model.restype = ctypes.c_int
     L.orc_gate.argtypes = [_f32p, _f32p, _i64, _i64, _i64, ctypes.c_float,
                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     L.orc_gate.restype = _i64
@@ -128,6 +130,18 @@ def normmap(hbits, tile, role):
     rc = lib().orc_normmap(hbits.reshape(-1), rows, cols, tile, role, nm.reshape(-1))
     if rc != 0:
         raise ValueError("orc_normmap: bad tile or dimensions")
+    return nm
+
+
+def normmap_ref16_model(hbits):
+    """Model of the reference's fp16 norm kernel (tile 32; fp16-rounded squares, fp16 column sums).
+    Parity unpinned by construction -- only for counting how many gate decisions could differ."""
+    hbits = np.ascontiguousarray(hbits, dtype=np.uint16)
+    rows, cols = hbits.shape
+    nm = np.empty((rows // 32, cols // 32), dtype=np.float32)
+    rc = lib().orc_normmap_ref16_model(hbits.reshape(-1), rows, cols, nm.reshape(-1))
+    if rc != 0:
+        raise ValueError("orc_normmap_ref16_model: dimensions must be multiples of 32")
     return nm
 
 

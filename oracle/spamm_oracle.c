@@ -214,6 +214,45 @@ ORC_API int orc_normmap(const uint16_t *H, int64_t rows, int64_t cols, int b, in
     return 0;
 }
 
+/* A MODEL of the reference's own fp16 norm kernel (unroll_get_Fnorm_FP16,
+ * cuSpAMM.cu:74-123; tile 32 only, as there), used by one CPU test to count how
+ * many gate decisions would differ from the clean fp32 norm above.  Not used
+ * for parity: what a WMMA unit does inside an fp16-accumulator product is not
+ * specified, so this function is PARITY UNPINNED by construction.
+ * Per 16 x 16 quarter of the tile (one warp, :93-94): every element is squared
+ * in fp32 and rounded to fp16 (:98-101); ones(16x16) x squares with an fp16
+ * accumulator gives the 16 column sums (:102) -- modelled as an exact sum of the
+ * 16 fp16 squares rounded once to fp16; the column sums times ones with an fp32
+ * accumulator gives their total (:109-112, element 0 is read at :116) --
+ * modelled as fp32 additions in ascending column order.  The four quarter
+ * totals are added in warp order and the square root taken in fp32 (:120). */
+ORC_API int orc_normmap_ref16_model(const uint16_t *H, int64_t rows, int64_t cols, float *nm) {
+    const int b = 32;
+    if (rows % b || cols % b) return -1;
+    const int64_t nbr = rows / b, nbc = cols / b;
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t I = 0; I < nbr; I++) {
+        for (int64_t J = 0; J < nbc; J++) {
+            float warp_total[4];
+            for (int w = 0; w < 4; w++) {
+                const uint16_t *T = H + (I * b + (w / 2) * 16) * cols + J * b + (w % 2) * 16;
+                float tot = 0.0f;
+                for (int c = 0; c < 16; c++) {
+                    double col = 0.0;                       /* exact: 16 fp16 values */
+                    for (int r = 0; r < 16; r++) {
+                        const float x = f16_bits_to_f32(T[(int64_t)r * cols + c]);
+                        col += (double)f16_bits_to_f32(f32_to_f16_bits(x * x));
+                    }
+                    tot = tot + f16_bits_to_f32(f32_to_f16_bits((float)col));
+                }
+                warp_total[w] = tot;
+            }
+            nm[I * nbc + J] = sqrtf(((warp_total[0] + warp_total[1]) + warp_total[2]) + warp_total[3]);
+        }
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------ gate */
 
 /* nA [nbM x nbK], nB [nbK x nbN] row-major.  keep(i,j,k) = nA[i,k]*nB[k,j] >= tau,

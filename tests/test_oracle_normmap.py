@@ -124,3 +124,32 @@ def test_rejects_bad_shapes(orc):
         orc.normmap(np.zeros((48, 64), dtype=np.uint16), 32, 0)
     with pytest.raises(ValueError):
         orc.normmap(np.zeros((64, 64), dtype=np.uint16), 16, 0)
+
+
+def test_reference_fp16_norm_model_and_the_gate_decisions_it_would_change(orc):
+    """The reference's fp16 norm kernel (cuSpAMM.cu:74-123) rounds every square to fp16 and sums
+    columns in an fp16 accumulator; the checker (and the GPU) use the clean fp32 norm.  A model of
+    that arithmetic shows how far apart the two are on BASELINE's first configuration (N = 1024,
+    A = B, exp(-0.5 d), tile 32, tau = 1e-4): the norms agree to ~1e-3 relative, and only products
+    within that distance of tau can be gated differently.  This is a report, not a parity pin."""
+    n, b, tau = 1024, 32, np.float32(1e-4)
+    X = orc.fill_decay(n, n, orc.decay_table("exp", n, 0.5), 1)
+    h = orc.f32_to_f16_bits(X)
+    clean_a, clean_b = orc.normmap(h, b, 0), orc.normmap(h, b, 1)
+    model = orc.normmap_ref16_model(h)
+    # closed forms hold for the model too: all-ones tile -> exactly 32, zeros -> 0
+    ones = orc.f32_to_f16_bits(np.ones((64, 64), dtype=np.float32))
+    assert np.all(orc.normmap_ref16_model(ones) == 32.0)
+    assert np.all(orc.normmap_ref16_model(np.zeros((32, 32), dtype=np.uint16)) == 0.0)
+    nz = clean_a > 1e-3                      # tiles whose squares are not lost to fp16 underflow
+    rel = np.abs(model[nz] - clean_a[nz]) / clean_a[nz]
+    assert rel.max() < 5e-3
+    # squares below 2^-24 vanish in fp16: far-off-diagonal tiles read as zero in the model
+    assert np.count_nonzero(model == 0) >= np.count_nonzero(clean_a == 0)
+    keep_clean = (clean_a[:, None, :] * clean_b.T[None, :, :]) >= tau       # [i, j, k]
+    keep_model = (model[:, None, :] * model.T[None, :, :]) >= tau
+    differ = int(np.count_nonzero(keep_clean != keep_model))
+    total = keep_clean.size
+    print("gate decisions that differ: %d of %d (%.4f %%), kept clean %d, kept model %d"
+          % (differ, total, 100.0 * differ / total, keep_clean.sum(), keep_model.sum()))
+    assert differ <= 0.005 * total
