@@ -420,27 +420,29 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
             }
         }
         if (threadIdx.x < 64 && deal == DEAL_BAND) {
-            // lane i holds the i-th super tile of the group, lane x the length of XCD x so far
+            // lane x < 8 holds the x-th super tile of the group and the length of XCD x so far; the
+            // 64 lanes compare all pairs at once (lane 8 i + j: i against j), so that the ranks of
+            // the eight super tiles (heaviest first) and of the eight XCDs (shortest first) are
+            // byte-wise popcounts of two ballots, and the match -- the super tile whose rank is the
+            // XCD's rank -- the lowest set bit of a third
             const int x = threadIdx.x;
+            const int pi = x >> 3, pj = x & 7;
             int load = 0, cnt = 0;
             const int ngroups = (n_ne + n_xcd - 1) / n_xcd;
             for (int g2 = 0; g2 < ngroups; g2++) {
                 const int r = g2 * n_xcd + x;
                 const int w = (x < n_xcd && r < n_ne) ? swork[r] : -1;           // -1: no super tile
-                int irank = 0, xrank = 0;       // my super tile among the group's, heaviest first; my XCD, shortest first
-#pragma unroll
-                for (int j = 0; j < MAX_XCD; j++) {
-                    const int wj = __builtin_amdgcn_readlane(w, j), lj = __builtin_amdgcn_readlane(load, j);
-                    irank += (wj > w) || (wj == w && j < x);
-                    xrank += (j < n_xcd) && ((lj < load) || (lj == load && j < x));
-                }
-                int mine = -1, wm = -1;         // the super tile whose rank is my XCD's rank
-#pragma unroll
-                for (int j = 0; j < MAX_XCD; j++) {
-                    const int rj = __builtin_amdgcn_readlane(irank, j), wj = __builtin_amdgcn_readlane(w, j);
-                    if (rj == xrank && j < n_xcd) { mine = j; wm = wj; }
-                }
-                if (x < n_xcd && wm > 0) {          // (the last group may have fewer super tiles than XCDs)
+                const int wi = __shfl(w, pi, 64), wj = __shfl(w, pj, 64);
+                const int li = __shfl(load, pi, 64), lj = __shfl(load, pj, 64);
+                const uint64_t heavier = __ballot((wj > wi) || (wj == wi && pj < pi));
+                const uint64_t shorter = __ballot(pj < n_xcd && ((lj < li) || (lj == li && pj < pi)));
+                const int irank_j = __builtin_popcountll((heavier >> (8 * pj)) & 0xffull);
+                const int xrank_i = __builtin_popcountll((shorter >> (8 * pi)) & 0xffull);
+                const uint64_t match = __ballot(pi < n_xcd && pj < n_xcd && irank_j == xrank_i);
+                const uint32_t mybyte = (uint32_t)((match >> (8 * (x & 7))) & 0xffull);     // lanes x < 8: row x
+                const int mine = mybyte ? __builtin_ctz(mybyte) : 0;
+                const int wm = __shfl(w, mine, 64);
+                if (x < n_xcd && mybyte && wm > 0) {   // (the last group may have fewer super tiles than XCDs)
                     sdeal[x * rounds + cnt] = (uint16_t)(g2 * n_xcd + mine);
                     cnt++;
                     load += wm;
