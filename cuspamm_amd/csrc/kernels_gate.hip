@@ -305,7 +305,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 // One workgroup; O(n^2) ranking over at most a few thousand super tiles.
 __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nMacN, int nSupN,
                                                 int n_super, int rounds, int n_xcd) {
-    extern __shared__ int swork[];               // [n_super] length, then [n_super] super tile origin by rank,
+    extern __shared__ __attribute__((aligned(16))) int swork[];               // [n_super] length, then [n_super] super tile origin by rank,
     int *srank_id = swork + n_super;             // then (greedy deal only) [n_xcd][rounds] rank of each XCD's r-th super tile
     uint16_t *sdeal = reinterpret_cast<uint16_t *>(srank_id + n_super);
     __shared__ unsigned long long total;
@@ -358,22 +358,57 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     const int deal = n_super > LPT_MAX_SUPER ? DEAL_SNAKE
                      : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT
                         : (n_ne <= BAND_DEAL_MAX && 5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
-    for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
-        const int w = swork[sid];
-        int rank = 0;
-        if (deal == DEAL_BAND) {
-            for (int j = 0; j < n_super; j++) {
-                const int wj = swork[j];
-                rank += ((wj > 0) > (w > 0)) || ((wj > 0) == (w > 0) && j < sid);
+    // rank = number of super tiles that come first: larger key, or equal key and smaller index;
+    // the key is the length, or in the band deal just "holds work".  n_super^2 comparisons: with
+    // few super tiles the j range is cut into `parts` pieces so that all 1024 threads take part
+    // (partial ranks meet in srank_id, used as a counter first); with many, a thread takes whole
+    // super tiles.
+    {
+        const bool band = deal == DEAL_BAND;
+        int parts = 1;
+        while (parts < 32 && n_super * parts * 2 <= (int)blockDim.x) parts *= 2;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) srank_id[sid] = 0;
+        __syncthreads();
+        const int chunk = (n_super + parts - 1) / parts;
+        // (two copies of the loop, one per key, so that the inner loop is a read, two compares and an add)
+        auto count_first = [&](auto key) {
+            if (parts == 1) {
+                for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
+                    const int w = key(swork[sid]);
+                    int rank = 0;
+                    for (int j = 0; j < n_super; j++) {
+                        const int kj = key(swork[j]);
+                        rank += (kj > w) || (kj == w && j < sid);
+                    }
+                    srank_id[sid] = rank;
+                }
+                return;
             }
-        } else {
-            for (int j = 0; j < n_super; j++) {
-                const int wj = swork[j];
-                rank += (wj > w) || (wj == w && j < sid);
+            for (int e = threadIdx.x; e < n_super * parts; e += blockDim.x) {
+                const int sid = e % n_super, part = e / n_super;
+                const int w = key(swork[sid]);
+                const int j1 = (part + 1) * chunk < n_super ? (part + 1) * chunk : n_super;
+                int rank = 0;
+                for (int j = part * chunk; j < j1; j++) {
+                    const int kj = key(swork[j]);
+                    rank += (kj > w) || (kj == w && j < sid);
+                }
+                if (rank) atomicAdd(&srank_id[sid], rank);
             }
+        };
+        if (band) count_first([](int v) { return (int)(v > 0); });
+        else count_first([](int v) { return v; });
+        __syncthreads();
+        int myrank[(LPT_MAX_SUPER + 1023) / 1024 > 8 ? (LPT_MAX_SUPER + 1023) / 1024 : 8];
+        int n = 0;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) myrank[n++ & 7] = srank_id[sid];
+        __syncthreads();
+        n = 0;
+        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
+            const int rank = myrank[n++ & 7];
+            srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
+            if (deal != DEAL_SNAKE) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
         }
-        srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
-        if (deal != DEAL_SNAKE) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
     }
     __syncthreads();
     if (deal != DEAL_SNAKE) {
