@@ -103,3 +103,40 @@ def test_noalloc_limits_and_flags(ctx):
     assert call(64, 64, 64, 64) == 0                               # x * x with tau 0: zeros
     ctx.synchronize()
     assert float(x.abs().max()) == 0.0
+
+
+# The callers this entry point is for: a HIP graph captures the multiply once and replays it on
+# changing inputs (mask and schedule are rebuilt on the device at every replay); eager multiplies
+# run between the replays and every replay is compared with one.
+def test_noalloc_multiply_replays_in_a_hip_graph(orc, ctx):
+    import torch
+    import cuspamm_amd as sp
+    M, K, N, tile, tau = 1024, 768, 1280, 64, 0.3
+    tab = orc.decay_table("exp", max(M, K, N), 0.01)
+    A0, B0 = orc.fill_decay(M, K, tab, 1), orc.fill_decay(K, N, tab, 2)
+    dA = torch.from_numpy(A0).cuda()
+    dB = torch.from_numpy(B0).cuda()
+    C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        gctx = sp.SpammContext(0)                     # bound to the side stream
+        gctx.multiply_noalloc(dA, dB, tile, tau, C)   # warm-up: kernels loaded before the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            gctx.multiply_noalloc(dA, dB, tile, tau, C, prune=True)
+    torch.cuda.synchronize()
+    for rep, scale in enumerate((1.0, 0.5, 3.0, 1.0)):
+        dA.copy_(torch.from_numpy(A0).cuda() * scale)                 # new inputs in the captured buffers
+        want = ctx.multiply(dA, dB, tile, tau).clone()                # eager work between the replays
+        want_mask = ctx.get_mask()
+        C.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(C, want), "replay %d" % rep
+        ref = orc.spamm((A0 * np.float32(scale)).astype(np.float32), B0, tile, tau)
+        assert np.array_equal(want_mask, ref["mask"])
+        err, nrm, _ = orc.frob_diff(C.cpu().numpy(), ref["C"])
+        assert err <= 1e-3 * nrm
+    gctx.close()
