@@ -10,7 +10,7 @@
 //
 //   spamm_main [--M m] [--K k] [--N n] [--tile 32|64|128] [--tau t | --ratio r | --tune r]
 //              [--gen exp|alg|ones] [--c c] [--v v] [--a-csv f --b-csv f | --a-mtx f --b-mtx f]
-//              [--testtime n] [--warmup n] [--check | --prune] [--device d]
+//              [--testtime n] [--warmup n] [--check | --prune] [--noalloc] [--device d]
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -37,7 +37,7 @@ int main(int argc, char **argv) {
     bool cv_given = false;
     std::string a_csv, b_csv, a_mtx, b_mtx;
     int testtime = 10, warmup = 5, device = 0;         // TESTTIME, WARMUP, para.h:4-5
-    bool check = false, prune = false;
+    bool check = false, prune = false, noalloc = false;
     for (int i = 1; i < argc; i++) {
         const std::string o = argv[i];
         auto val = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };
@@ -60,6 +60,7 @@ int main(int argc, char **argv) {
         else if (o == "--device") device = atoi(val());
         else if (o == "--check") check = true;
         else if (o == "--prune") prune = true;
+        else if (o == "--noalloc") noalloc = true;        // the timed multiplies run in the library's fixed workspace
         else { fprintf(stderr, "spamm_main: unknown option %s\n", o.c_str()); return 2; }
     }
     if (gen == "exp" && !cv_given) { c = 1.0f; v = 0.1f; }    // getDecayMatrixExp(h, 1, 0.1, ...), cuSpAMM.cu:426-427
@@ -126,7 +127,8 @@ int main(int argc, char **argv) {
     spamm_stats st;
     memset(&st, 0, sizeof(st));
     for (int i = 0; i < testtime; i++) {
-        if ((rc = spamm_multiply(ctx, &p, dA, dB, dC))) return fail("spamm_multiply", rc);
+        if ((rc = noalloc ? spamm_multiply_noalloc(ctx, &p, dA, dB, dC) : spamm_multiply(ctx, &p, dA, dB, dC)))
+            return fail(noalloc ? "spamm_multiply_noalloc" : "spamm_multiply", rc);
         if ((rc = spamm_get_stats(ctx, &st))) return fail("spamm_get_stats", rc);
         if (i > warmup) sum += st.ms_total * 1e-3;       // cuSpAMM.cu:548
     }

@@ -57,3 +57,19 @@ def test_driver_pads_and_tunes(orc):
 def test_driver_rejects_bad_arguments():
     proc = subprocess.run([MAIN, "--tile", "48"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     assert proc.returncode == 2 and "tile must be" in proc.stdout
+
+
+def test_driver_in_the_fixed_workspace():
+    # --noalloc: the timed multiplies go through spamm_multiply_noalloc; same printed counts and norms
+    args = ["--M", 1024, "--K", 768, "--N", 1280, "--tile", 64, "--gen", "exp", "--c", 1.0, "--v", 0.98, "--tau", 0.05,
+            "--testtime", 3, "--warmup", 0, "--check"]
+    plain, fixed = _run(args), _run(args + ["--noalloc"])
+    pick = lambda out: (re.search(r"valid products=(\d+) of (\d+)", out).groups(),
+                        re.search(r"\|C_dense-C\|_F=(\S+) \|C_dense\|_F=(\S+) \|C\|_F=(\S+) bound=(\S+)", out).groups())
+    assert pick(plain) == pick(fixed)
+    kept, total = map(int, pick(fixed)[0])
+    assert 0 < kept < total
+    # a problem beyond the fixed workspace is refused with the library's message
+    proc = subprocess.run([MAIN, "--M", "8192", "--K", "8192", "--N", "8192", "--tile", "64", "--tau", "1", "--testtime", "2",
+                           "--warmup", "0", "--noalloc"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode != 0 and "fixed workspace" in proc.stdout, proc.stdout

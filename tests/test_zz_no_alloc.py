@@ -79,6 +79,28 @@ def test_noalloc_a_equals_b(orc, ctx):
     _check_against(ctx, orc, got, orc.spamm(A, A, 32, 1e-2), "noalloc A = B")
 
 
+def test_noalloc_at_the_workspace_limit(orc, ctx):
+    # 3072^3 needs 36 MiB of fp16 copies plus lists: the largest cube that fits the 40 MiB array
+    import torch
+    n = 3072
+    tab = orc.decay_table("exp", n, 0.004)
+    dA = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    dB = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    ctx.fill_decay(dA, tab, 1)
+    ctx.fill_decay(dB, tab, 2)
+    for tile in (32, 128):
+        ctx.normmap_f32(1, dB, tile)
+        ctx.normmap_f32(0, dA, tile)
+        tau, ach = ctx.tau_for_ratio(0.15)
+        want = ctx.multiply(dA, dB, tile, tau, prune=True).clone()
+        want_mask, want_counts = ctx.get_mask(), ctx.get_counts()
+        got = torch.full((n, n), float("nan"), dtype=torch.float32, device="cuda")
+        ctx.multiply_noalloc(dA, dB, tile, tau, got, prune=True)
+        assert np.array_equal(ctx.get_mask(), want_mask) and np.array_equal(ctx.get_counts(), want_counts)
+        assert torch.equal(got, want)
+        assert abs(ctx.get_stats().kept_products / (n // tile) ** 3 - ach) < 1e-9
+
+
 def test_noalloc_limits_and_flags(ctx):
     import ctypes
     import torch
