@@ -358,32 +358,24 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     const int deal = n_super > LPT_MAX_SUPER ? DEAL_SNAKE
                      : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT
                         : (n_ne <= BAND_DEAL_MAX && 5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
-    // rank = number of super tiles that come first: larger key, or equal key and smaller index;
-    // the key is the length, or in the band deal just "holds work".  n_super^2 comparisons: with
-    // few super tiles the j range is cut into `parts` pieces so that all 1024 threads take part
-    // (partial ranks meet in srank_id, used as a counter first); with many, a thread takes whole
-    // super tiles.
-    {
+    // Ranking: larger key first, equal keys by smaller index; the key is the length, or in the
+    // band deal just "holds work".  srank_id[rank] becomes the super tile's origin.
+    //   up to RANK_SORT_MIN super tiles: rank = number of super tiles that come first, n_super^2
+    //   comparisons with the j range cut into `parts` pieces so that all 1024 threads take part
+    //   (partial ranks meet in srank_id, used as a counter first);
+    //   beyond: a bitonic sort of the indices in LDS (padded to a power of two with indices
+    //   >= n_super, which sort last): log^2 steps of one compare-exchange per thread instead of
+    //   n_super comparisons per super tile on this one CU (150 us at 2048 super tiles).
+    constexpr int RANK_SORT_MIN = 512;
+    if (n_super <= RANK_SORT_MIN) {
         const bool band = deal == DEAL_BAND;
-        int parts = 1;
+        int parts = 2;
         while (parts < 32 && n_super * parts * 2 <= (int)blockDim.x) parts *= 2;
         for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) srank_id[sid] = 0;
         __syncthreads();
         const int chunk = (n_super + parts - 1) / parts;
         // (two copies of the loop, one per key, so that the inner loop is a read, two compares and an add)
         auto count_first = [&](auto key) {
-            if (parts == 1) {
-                for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
-                    const int w = key(swork[sid]);
-                    int rank = 0;
-                    for (int j = 0; j < n_super; j++) {
-                        const int kj = key(swork[j]);
-                        rank += (kj > w) || (kj == w && j < sid);
-                    }
-                    srank_id[sid] = rank;
-                }
-                return;
-            }
             for (int e = threadIdx.x; e < n_super * parts; e += blockDim.x) {
                 const int sid = e % n_super, part = e / n_super;
                 const int w = key(swork[sid]);
@@ -399,15 +391,39 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         if (band) count_first([](int v) { return (int)(v > 0); });
         else count_first([](int v) { return v; });
         __syncthreads();
-        int myrank[(LPT_MAX_SUPER + 1023) / 1024 > 8 ? (LPT_MAX_SUPER + 1023) / 1024 : 8];
-        int n = 0;
-        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) myrank[n++ & 7] = srank_id[sid];
+        const int sid = threadIdx.x;              // n_super <= RANK_SORT_MIN < blockDim.x: one super tile per thread
+        const int rank = sid < n_super ? srank_id[sid] : 0;
         __syncthreads();
-        n = 0;
-        for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) {
-            const int rank = myrank[n++ & 7];
+        if (sid < n_super) {
             srank_id[rank] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);   // first macro tile row, column
             if (deal != DEAL_SNAKE) sdeal[sid] = (uint16_t)rank;       // parked: rank of super tile sid (read back below)
+        }
+    } else {
+        int np2 = 2 * RANK_SORT_MIN;
+        while (np2 < n_super) np2 <<= 1;
+        int *sidx = srank_id;                     // [np2]: runs into sdeal's space, which is not in use yet
+        for (int i = threadIdx.x; i < np2; i += blockDim.x) sidx[i] = i;
+        __syncthreads();
+        auto sort_by = [&](auto key) {
+            for (int k = 2; k <= np2; k <<= 1)
+                for (int j = k >> 1; j > 0; j >>= 1) {
+                    for (int t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
+                        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), l = i | j;
+                        const int a = sidx[i], b = sidx[l];
+                        const int ka = a < n_super ? key(swork[a]) : -1, kb = b < n_super ? key(swork[b]) : -1;
+                        const bool a_first = ka > kb || (ka == kb && a < b);
+                        if (a_first != ((i & k) == 0)) { sidx[i] = b; sidx[l] = a; }
+                    }
+                    __syncthreads();
+                }
+        };
+        if (deal == DEAL_BAND) sort_by([](int v) { return (int)(v > 0); });
+        else sort_by([](int v) { return v; });
+        // sidx[rank] = super tile; every thread turns its own slots into origins
+        for (int r = threadIdx.x; r < n_super; r += blockDim.x) {
+            const int sid = sidx[r];
+            srank_id[r] = ((sid / nSupN) * SUPER_M) << 16 | ((sid % nSupN) * SUPER_N);
+            if (deal != DEAL_SNAKE) sdeal[sid] = (uint16_t)r;
         }
     }
     __syncthreads();

@@ -112,8 +112,13 @@ inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
     const int64_t nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
     const size_t n_super = (size_t)(((nMacM + SUPER_M - 1) / SUPER_M) * ((nMacN + SUPER_N - 1) / SUPER_N));
     // length + origin by rank, and for the greedy deal a table of at most MAX_XCD x rounds (or
-    // n_super parked ranks) 16-bit entries
-    return n_super * 2 * sizeof(int) + (n_super <= (size_t)LPT_MAX_SUPER ? (n_super + 2 * MAX_XCD) * sizeof(uint16_t) * 2 : 0);
+    // n_super parked ranks) 16-bit entries; beyond 512 super tiles the ranking sorts indices
+    // padded to a power of two in the second array's place
+    size_t np2 = 1024;
+    while (np2 < n_super) np2 *= 2;
+    const size_t tables = n_super * 2 * sizeof(int) + (n_super <= (size_t)LPT_MAX_SUPER ? (n_super + 2 * MAX_XCD) * sizeof(uint16_t) * 2 : 0);
+    const size_t sorting = n_super > 512 ? (n_super + np2) * sizeof(int) : 0;
+    return tables > sorting ? tables : sorting;
 }
 inline size_t order_lds_limit() { return 64 * 1024; }
 hipError_t gate_init();   // one-time kernel attribute set-up

@@ -59,6 +59,20 @@ def test_extreme_aspect_ratios(orc, ctx, M, K, N, tile):
     assert 0 < ref["kept"]
 
 
+def test_more_than_512_super_tiles_of_c(orc, ctx):
+    # 520 super tiles (not a power of two): the schedule ranks them by sorting; B's non-zero column
+    # range is cut so that all of them, 40 % and 10 % hold work -- one case per way of dealing
+    M, K, tile = 256, 64, 64
+    N = 520 * 8 * 256
+    tab = orc.decay_table("exp", N, 0.0)
+    A = orc.fill_decay(M, K, tab, 1)
+    B = orc.fill_decay(K, N, tab, 2)
+    for frac in (1.0, 0.4, 0.1):
+        B[:, int(N * frac):] = 0.0
+        ref = _check(orc, ctx, A, B, tile, 1e-30)
+        assert ref["kept"] == (M // tile) * (int(N * frac) // tile)
+
+
 def test_scattered_sparsity_pattern(orc, ctx):
     # no band structure at all: random tiles zeroed, so k lists are ragged and macro tiles mixed
     rng = np.random.default_rng(7)
