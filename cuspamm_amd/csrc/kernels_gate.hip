@@ -597,8 +597,11 @@ hipError_t gate_init() {
                                  (int)gate_lds_limit())) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<4>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                  (int)gate_lds_limit())) != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)gate_lds_limit());
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)gate_lds_limit())) != hipSuccess) return e;
+    // k_order: its tables may take order_lds_limit() on top of a few static bytes
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_order), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)order_lds_limit());
 }
 
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,

@@ -214,6 +214,27 @@ def test_gate_on_random_maps_with_ragged_k(orc, ctx):
             assert ctx.get_stats().kept_products == total
 
 
+def test_gate_at_the_most_super_tiles_of_c(orc, ctx):
+    # 64 x 128 = 8192 super tiles of C (tile 128: 512 x 2048 tiles) fill the schedule kernel's
+    # tables to their limit; one tile more in either direction is refused, not mis-scheduled
+    import cuspamm_amd as sp
+    rng = np.random.default_rng(11)
+    nbM, nbK, nbN, tile = 512, 2, 2048, 128
+    nA = np.abs(rng.normal(size=(nbM, nbK))).astype(np.float32)
+    nB = np.abs(rng.normal(size=(nbK, nbN))).astype(np.float32)
+    ctx.set_normmaps(nA, nB, tile)
+    ctx.gate(1.0)
+    total, counts, _, mask = orc.gate(nA, nB, 1.0, want_klist=False)
+    assert np.array_equal(ctx.get_counts(), counts)
+    assert np.array_equal(ctx.get_mask(), mask)
+    assert ctx.get_stats().kept_products == total
+    for shape in ((nbM + 1, nbN), (nbM, nbN + 1)):
+        ctx.set_normmaps(np.ones((shape[0], nbK), np.float32), np.ones((nbK, shape[1]), np.float32), tile)
+        with pytest.raises(sp.SpammError) as e:
+            ctx.gate(1.0)
+        assert e.value.code == -1                             # invalid argument: size limit
+
+
 def test_error_vs_fp64_dense_and_bound(orc, ctx):
     tab = orc.decay_table("exp", 1024, 0.01)
     A = orc.fill_decay(1024, 1024, tab, 1)

@@ -59,18 +59,23 @@ def test_extreme_aspect_ratios(orc, ctx, M, K, N, tile):
     assert 0 < ref["kept"]
 
 
-def test_more_than_512_super_tiles_of_c(orc, ctx):
-    # 520 super tiles (not a power of two): the schedule ranks them by sorting; B's non-zero column
-    # range is cut so that all of them, 40 % and 10 % hold work -- one case per way of dealing
-    M, K, tile = 256, 64, 64
-    N = 520 * 8 * 256
+@pytest.mark.parametrize("M,n_sup_n,percents", [(256, 520, (100, 40, 10)), (1088, 1030, (100, 30))])
+def test_more_than_512_super_tiles_of_c(orc, ctx, M, n_sup_n, percents):
+    # beyond 512 super tiles the schedule ranks them by sorting indices padded to a power of two:
+    # 1 x 520 -> 1024, and 2 x 1030 = 2060 -> 4096 (M = 1088 is five macro tile rows, the fifth
+    # starts a second row of super tiles; 9 GB of C).  B's non-zero column range is cut so that all,
+    # 40 % and 10 % of the 520 super tiles hold work -- one case per way of dealing; beyond 2048
+    # super tiles there is one way only
+    K, tile = 64, 64
+    N = n_sup_n * 8 * 256
     tab = orc.decay_table("exp", N, 0.0)
     A = orc.fill_decay(M, K, tab, 1)
     B = orc.fill_decay(K, N, tab, 2)
-    for frac in (1.0, 0.4, 0.1):
-        B[:, int(N * frac):] = 0.0
+    for percent in percents:
+        cut = N * percent // 100          # a multiple of the tile size
+        B[:, cut:] = 0.0
         ref = _check(orc, ctx, A, B, tile, 1e-30)
-        assert ref["kept"] == (M // tile) * (int(N * frac) // tile)
+        assert ref["kept"] == (M // tile) * (cut // tile)
 
 
 def test_scattered_sparsity_pattern(orc, ctx):
