@@ -35,6 +35,8 @@ WORKLOADS = {
     # short distance) gives the smallest positive norm product as tau: the largest kept fraction.
     "headline": (16384, 64, "exp", 0.003, 0.10, None),
     "headline_literal": (16384, 64, "exp", 0.1, 0.10, None),     # the decay rate as written: 10 % unreachable
+    "headline_b32": (16384, 32, "exp", 0.003, 0.10, None),       # the reference's tile size (main.h:32 LoNum)
+    "headline_b128": (16384, 128, "exp", 0.003, 0.10, None),
     "cfg2": (8192, 64, "exp", 0.01, 0.10, None),
     "cfg2_literal": (8192, 64, "exp", 0.1, 0.10, None),          # as written: 10 % unreachable
     "cfg3_05": (16384, 64, "alg", 0.0, 0.05, None),
