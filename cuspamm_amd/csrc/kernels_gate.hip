@@ -20,6 +20,8 @@
 // The reference's compacted per-tile list (offset[], :315-325) is the bitmap's
 // set bits in ascending order; nothing downstream reads it, so it is produced
 // from the bitmap only when asked for (k_klist).
+#include <type_traits>
+
 #include "spamm_internal.h"
 
 namespace spamm {
@@ -43,9 +45,18 @@ __device__ __forceinline__ uint64_t transpose64(uint64_t x, int lane) {
     return x;
 }
 
-// v[lane idx] = s for a wave-uniform s; idx must fold to a constant (unrolled loops)
-__device__ __forceinline__ void set_lane(int &v, uint32_t s, int idx) {
-    asm("v_writelane_b32 %0, %1, %2" : "+v"(v) : "s"(s), "n"(idx));
+// lo[lane idx] = low word, hi[lane idx] = high word of a wave-uniform 64-bit m; idx must fold to
+// a constant (unrolled loops).  On gfx90a and later a VALU instruction that reads an SGPR needs
+// two wait states after the VALU instruction that wrote it (here: the compare behind the ballot).
+// The compiler inserts them only around instructions it can see, not around inline assembly, so
+// the s_nop is part of it.
+__device__ __forceinline__ void set_lane2(int &lo, int &hi, uint64_t m, int idx) {
+    // (readfirstlane: under register pressure the compiler may hold the uniform words in VGPRs)
+    const int mlo = __builtin_amdgcn_readfirstlane((int)(uint32_t)m);
+    const int mhi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(m >> 32));
+    asm("s_nop 1\n\tv_writelane_b32 %0, %2, %4\n\tv_writelane_b32 %1, %3, %4"
+        : "+v"(lo), "+v"(hi)
+        : "s"(mlo), "s"(mhi), "n"(idx));
 }
 
 template <int MT>
@@ -58,14 +69,21 @@ struct GateCfg {
     static constexpr uint64_t FULL = NT == 64 ? ~0ull : ((1ull << NT) - 1ull);
 };
 
-template <int MT>
-__global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int nMacN, float tau) {
+template <int MT, bool ONE>
+__global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int nMacN, float tau, int cw_arg) {
     using G = GateCfg<MT>;
     constexpr int NT = G::NT, NTP = G::NTP, BT = G::BT;
     extern __shared__ uint64_t smem[];
     const int words = (nbK + 63) >> 6;
-    uint64_t *lmask = smem;                                  // [words][NTP]: tile bitmaps, later transposed in place
-    uint64_t *luf = smem + (size_t)words * NTP;              // [words][2]: union word, kept-by-all word
+    // LDS holds the tile bitmaps of `cw` 64-k words at a time (cw = words unless K / tile is so
+    // large that a macro tile's bitmaps exceed a CU's LDS: then the k range is walked in chunks,
+    // twice -- once to count, once to place the list entries -- and the bitmaps of a chunk are
+    // recomputed for the second walk); the per-word summaries below cover all words.  ONE: the
+    // instantiation for cw = words, straight-line code without the chunk loop.
+    constexpr bool one_chunk = ONE;
+    const int cw = ONE ? words : cw_arg;
+    uint64_t *lmask = smem;                                  // [cw][NTP]: tile bitmaps, later transposed in place
+    uint64_t *luf = smem + (size_t)cw * NTP;                 // [words][2]: union word, kept-by-all word
     int *wfull = reinterpret_cast<int *>(luf + 2 * (size_t)words);   // [words + 1] prefix of full entries
     int *wpart = wfull + (words + 1);                        // [words + 1] prefix of partial entries
 
@@ -81,8 +99,8 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     struct Item {
         float pa[BT], pb[BT];
     };
-    auto load_item = [&](int item, Item &it) {
-        const int q = item % G::NQ, w = item / G::NQ;
+    auto load_item = [&](int w0, int item, Item &it) {
+        const int q = item % G::NQ, w = w0 + item / G::NQ;
         const int k = w * 64 + lane;
         const int kc = k < nbK ? k : nbK - 1;
 #pragma unroll
@@ -98,8 +116,8 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     };
     // whole macro tile inside the matrix: only the last k word may need masking
     const bool interior = (mi + 1) * MT <= nbM && (mj + 1) * MT <= nbN;
-    auto gate_item = [&](int item, const Item &it) {
-        const int q = item % G::NQ, w = item / G::NQ;
+    auto gate_item = [&](int w0, int item, const Item &it) {
+        const int q = item % G::NQ, wl = item / G::NQ, w = w0 + wl;
         const int ti0 = (q / G::QD) * BT, tj0 = (q % G::QD) * BT;
         int mlo = 0, mhi = 0;                 // lane a*BT+b collects the word of tile (a, b)
         if (interior && (w + 1) * 64 <= nbK) {
@@ -108,8 +126,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
 #pragma unroll
                 for (int b = 0; b < BT; b++) {
                     const uint64_t m = __ballot(it.pa[a] * it.pb[b] >= tau);
-                    set_lane(mlo, (uint32_t)m, a * BT + b);
-                    set_lane(mhi, (uint32_t)(m >> 32), a * BT + b);
+                    set_lane2(mlo, mhi, m, a * BT + b);
                 }
         } else {
             const uint64_t kmask = __ballot(w * 64 + lane < nbK);
@@ -121,75 +138,123 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
                     const uint64_t inside =
                         0ull - (uint64_t)((mi * MT + ti0 + a < nbM) & (mj * MT + tj0 + b < nbN));
                     const uint64_t m = __ballot(it.pa[a] * it.pb[b] >= tau) & kmask & inside;
-                    set_lane(mlo, (uint32_t)m, a * BT + b);
-                    set_lane(mhi, (uint32_t)(m >> 32), a * BT + b);
+                    set_lane2(mlo, mhi, m, a * BT + b);
                 }
         }
         if (lane < BT * BT)
-            lmask[(size_t)w * NTP + (ti0 + lane / BT) * MT + tj0 + lane % BT] =
+            lmask[(size_t)wl * NTP + (ti0 + lane / BT) * MT + tj0 + lane % BT] =
                 ((uint64_t)(uint32_t)mhi << 32) | (uint32_t)mlo;
     };
-    const int n_items = G::NQ * words;
-    for (int it0 = wave; it0 < n_items; it0 += 8) {
-        const int it1 = it0 + 4;
-        Item i0, i1;
-        load_item(it0, i0);
-        if (it1 < n_items) load_item(it1, i1);
-        gate_item(it0, i0);
-        if (it1 < n_items) gate_item(it1, i1);
-    }
-    __syncthreads();
-
-    // ---- phase 2a: per-tile counts, the macro tile's kept-product total, bitmaps to memory
-    int work = 0;
-    if (wave == 0) {
-        int cnt = 0;
-        if (lane < NT) {
-            for (int w = 0; w < words; w++) cnt += __builtin_popcountll(lmask[(size_t)w * NTP + lane]);
-            const int i = mi * MT + lane / MT, j = mj * MT + lane % MT;
-            if (i < nbM && j < nbN) g.counts[(int64_t)i * nbN + j] = cnt;
+    auto build_bitmaps = [&](int w0, int cwn) {
+        const int n_items = G::NQ * cwn;
+        for (int it0 = wave; it0 < n_items; it0 += 8) {
+            const int it1 = it0 + 4;
+            Item i0, i1;
+            load_item(w0, it0, i0);
+            if (it1 < n_items) load_item(w0, it1, i1);
+            gate_item(w0, it0, i0);
+            if (it1 < n_items) gate_item(w0, it1, i1);
         }
-        work = cnt;
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) work += __shfl_xor(work, off, 64);
-    }
-    const float inv_words = 1.0f / (float)words;     // e < 2^16, words <= 1024: the quotient below is exact
-    for (int e = threadIdx.x; e < NT * words; e += 256) {
-        const int t = (int)(((float)e + 0.5f) * inv_words), w = e - t * words;
-        const int i = mi * MT + t / MT, j = mj * MT + t % MT;
-        if (i < nbM && j < nbN) g.mask[((int64_t)i * nbN + j) * words + w] = lmask[(size_t)w * NTP + t];
-    }
-    __syncthreads();
-
+    };
     // ---- phase 2b: transpose every word in place: entry b of word w becomes the set of tiles
     // (bit t = tile t of the macro tile) that keep k = 64 w + b, NTP bits wide
-    auto tile_bits = [&](int w, int b) -> uint64_t {
-        if constexpr (NTP == 64) return lmask[(size_t)w * 64 + b];
-        else if constexpr (NTP == 16) return reinterpret_cast<const uint16_t *>(lmask + (size_t)w * 16)[b];
-        else return reinterpret_cast<const uint8_t *>(lmask + (size_t)w * 8)[b];
+    auto tile_bits = [&](int wl, int b) -> uint64_t {
+        if constexpr (NTP == 64) return lmask[(size_t)wl * 64 + b];
+        else if constexpr (NTP == 16) return reinterpret_cast<const uint16_t *>(lmask + (size_t)wl * 16)[b];
+        else return reinterpret_cast<const uint8_t *>(lmask + (size_t)wl * 8)[b];
     };
-    for (int w = wave; w < words; w += 4) {
-        const uint64_t row = lane < NT ? lmask[(size_t)w * NTP + lane] : 0ull;
-        const uint64_t bits = transpose64(row, lane);
-        const uint64_t u = __ballot(bits != 0ull), f = __ballot(bits == G::FULL);
-        // the wave has read all rows of the word before any lane writes its column
-        if constexpr (NTP == 64) lmask[(size_t)w * 64 + lane] = bits;
-        else if constexpr (NTP == 16) reinterpret_cast<uint16_t *>(lmask + (size_t)w * 16)[lane] = (uint16_t)bits;
-        else reinterpret_cast<uint8_t *>(lmask + (size_t)w * 8)[lane] = (uint8_t)bits;
-        if (lane == 0) {
-            luf[2 * w] = u;
-            luf[2 * w + 1] = f;
-            wfull[w + 1] = __builtin_popcountll(f);
-            wpart[w + 1] = __builtin_popcountll(u & ~f);
+    auto transpose_words = [&](int w0, int cwn, bool record) {
+        for (int wl = wave; wl < cwn; wl += 4) {
+            const uint64_t row = lane < NT ? lmask[(size_t)wl * NTP + lane] : 0ull;
+            const uint64_t bits = transpose64(row, lane);
+            const uint64_t u = __ballot(bits != 0ull), f = __ballot(bits == G::FULL);
+            // the wave has read all rows of the word before any lane writes its column
+            if constexpr (NTP == 64) lmask[(size_t)wl * 64 + lane] = bits;
+            else if constexpr (NTP == 16) reinterpret_cast<uint16_t *>(lmask + (size_t)wl * 16)[lane] = (uint16_t)bits;
+            else reinterpret_cast<uint8_t *>(lmask + (size_t)wl * 8)[lane] = (uint8_t)bits;
+            if (record && lane == 0) {
+                const int w = w0 + wl;
+                luf[2 * w] = u;
+                luf[2 * w + 1] = f;
+                wfull[w + 1] = __builtin_popcountll(f);
+                wpart[w + 1] = __builtin_popcountll(u & ~f);
+            }
         }
-    }
+    };
+
+    int cnt = 0;                               // wave 0, lane < NT: kept k of tile `lane`
+    int n_full = 0, n_part = 0, rot_f = 0, rot_p = 0;
+    // One walk over the k chunks; `pass` is a compile-time tag: 0 counts, 1 places.
+    auto walk = [&](auto pass_tag) {
+        constexpr int pass = decltype(pass_tag)::value;
+        int w0 = 0;
+        do {
+            const int cwn = words - w0 < cw ? words - w0 : cw;
+            if constexpr (pass == 0 || !one_chunk) {
+                build_bitmaps(w0, cwn);
+                __syncthreads();
+            }
+            if constexpr (pass == 0) {
+                // ---- phase 2a: per-tile counts and the bitmaps to memory
+                if (wave == 0 && lane < NT)
+                    for (int wl = 0; wl < cwn; wl++) cnt += __builtin_popcountll(lmask[(size_t)wl * NTP + lane]);
+                const float inv_words = 1.0f / (float)cwn;     // e < 2^16, cwn <= 1024: the quotient below is exact
+                for (int e = threadIdx.x; e < NT * cwn; e += 256) {
+                    const int t = (int)(((float)e + 0.5f) * inv_words), wl = e - t * cwn;
+                    const int i = mi * MT + t / MT, j = mj * MT + t % MT;
+                    if (i < nbM && j < nbN) g.mask[((int64_t)i * nbN + j) * words + w0 + wl] = lmask[(size_t)wl * NTP + t];
+                }
+                __syncthreads();
+            }
+            if constexpr (pass == 0 || !one_chunk) {
+                transpose_words(w0, cwn, pass == 0);
+                __syncthreads();
+            }
+            if constexpr (pass == 1) {
+                // ---- phase 2c: union list with per-tile bits.  Entries whose k is kept by every
+                // tile of the macro tile ("full") come first, then the partial ones, each group
+                // in ascending k rotated to the anchor: the GEMM runs a branch-free loop over the
+                // first group.
+                const int k1 = (w0 + cwn) * 64 < nbK ? (w0 + cwn) * 64 : nbK;
+                for (int k = w0 * 64 + threadIdx.x; k < k1; k += 256) {
+                    const int w = k >> 6, b = k & 63;
+                    const uint64_t bits = tile_bits(w - w0, b);
+                    if (bits != 0ull) {
+                        const uint64_t u = luf[2 * w], f = luf[2 * w + 1];
+                        const uint64_t below = (1ull << b) - 1ull;
+                        int pos;
+                        if (bits == G::FULL) {
+                            pos = wfull[w] + __builtin_popcountll(f & below) - rot_f;
+                            if (pos < 0) pos += n_full;
+                        } else {
+                            pos = wpart[w] + __builtin_popcountll(u & ~f & below) - rot_p;
+                            if (pos < 0) pos += n_part;
+                            pos += n_full;
+                        }
+                        uint32_t need = 0;
+#pragma unroll
+                        for (int a = 0; a < MT; a++) {
+                            const uint32_t rowbits = (uint32_t)(bits >> (a * MT)) & ((1u << MT) - 1u);
+                            if (rowbits) need |= 1u << a;
+                            need |= rowbits << 8;
+                        }
+                        MacroEntry en;
+                        en.k = (uint32_t)k;
+                        en.need = need;
+                        en.mask_lo = (uint32_t)bits;
+                        en.mask_hi = (uint32_t)(bits >> 32);
+                        g.macro_list[(int64_t)macro * nbK + pos] = en;
+                    }
+                }
+                if constexpr (!one_chunk) __syncthreads();     // the next chunk's bitmaps overwrite these
+            }
+            w0 += cw;
+        } while (!ONE && w0 < words);
+    };
+    walk(std::integral_constant<int, 0>{});
+    // ---- between the walks: inclusive scans over the words give each word's offset in its group
     if (threadIdx.x == 0) { wfull[0] = 0; wpart[0] = 0; }
     __syncthreads();
-
-    // ---- phase 2c: union list with per-tile bits.  Entries whose k is kept by
-    // every tile of the macro tile ("full") come first, then the partial ones,
-    // each group in ascending k: the GEMM runs a branch-free loop over the
-    // first group.  Inclusive scans over the words give each word's offset.
     if (words < 64) {
         if (wave == 0) {
             int vf = lane <= words ? wfull[lane] : 0, vp = lane <= words ? wpart[lane] : 0;
@@ -221,13 +286,12 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
             __syncthreads();
         }
     }
-    const int n_full = wfull[words];
-    const int n_part = wpart[words];
+    n_full = wfull[words];
+    n_part = wpart[words];
     // Each group is rotated to start at an anchor k shared by the whole super
     // tile (the k where its diagonal would sit): the workgroups of a super
     // tile run together on one XCD, and walking k from a common start keeps
     // them on the same A row panels and B column panels at the same time.
-    int rot_f = 0, rot_p = 0;              // entries of each group below the anchor
     {
         const int sm = mi / SUPER_M, sn = mj / SUPER_N;
         const float ic = ((sm * SUPER_M + 0.5f * SUPER_M) * MT) / (float)nbM;
@@ -238,38 +302,20 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         const int wa = anchor >> 6, ba = anchor & 63;
         const uint64_t u = luf[2 * wa], f = luf[2 * wa + 1];
         const uint64_t below = (1ull << ba) - 1ull;
-        rot_f = wfull[wa] + __builtin_popcountll(f & below);
+        rot_f = wfull[wa] + __builtin_popcountll(f & below);     // entries of each group below the anchor
         rot_p = wpart[wa] + __builtin_popcountll(u & ~f & below);
     }
-    for (int k = threadIdx.x; k < nbK; k += 256) {
-        const int w = k >> 6, b = k & 63;
-        const uint64_t bits = tile_bits(w, b);
-        if (bits != 0ull) {
-            const uint64_t u = luf[2 * w], f = luf[2 * w + 1];
-            const uint64_t below = (1ull << b) - 1ull;
-            int pos;
-            if (bits == G::FULL) {
-                pos = wfull[w] + __builtin_popcountll(f & below) - rot_f;
-                if (pos < 0) pos += n_full;
-            } else {
-                pos = wpart[w] + __builtin_popcountll(u & ~f & below) - rot_p;
-                if (pos < 0) pos += n_part;
-                pos += n_full;
-            }
-            uint32_t need = 0;
-#pragma unroll
-            for (int a = 0; a < MT; a++) {
-                const uint32_t rowbits = (uint32_t)(bits >> (a * MT)) & ((1u << MT) - 1u);
-                if (rowbits) need |= 1u << a;
-                need |= rowbits << 8;
-            }
-            MacroEntry en;
-            en.k = (uint32_t)k;
-            en.need = need;
-            en.mask_lo = (uint32_t)bits;
-            en.mask_hi = (uint32_t)(bits >> 32);
-            g.macro_list[(int64_t)macro * nbK + pos] = en;
+    walk(std::integral_constant<int, 1>{});
+    // per-tile counts and the macro tile's kept-product total
+    int work = 0;
+    if (wave == 0) {
+        if (lane < NT) {
+            const int i = mi * MT + lane / MT, j = mj * MT + lane % MT;
+            if (i < nbM && j < nbN) g.counts[(int64_t)i * nbN + j] = cnt;
         }
+        work = cnt;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) work += __shfl_xor(work, off, 64);
     }
     if (threadIdx.x == 0) {
         g.macro_count[2 * macro] = n_full + n_part;
@@ -583,39 +629,59 @@ hipError_t launch_klist(const uint64_t *mask, uint16_t *klist, int64_t n_tiles, 
     return hipGetLastError();
 }
 
-size_t gate_lds_bytes(int tile, int64_t nbK) {
+// A macro tile's bitmaps take words * NTP * 8 bytes of LDS (tile 32: 512 bytes per 64 k tiles)
+// beside 24 bytes of summaries per word; what does not fit a CU's LDS is walked in chunks of
+// gate_chunk_words() words; `cap` > 0 (a context's developer knob) forces smaller chunks so that
+// ordinary shapes take the chunked path.
+static size_t gate_fixed_bytes(size_t words) { return words * 16 + 2 * (words + 1) * 4; }
+
+int gate_chunk_words(int tile, int64_t nbK, int cap) {
     const int MT = macro_dim(tile);
     const size_t ntp = MT * MT < 8 ? 8 : MT * MT;
     const size_t words = (size_t)((nbK + 63) / 64);
-    return ntp * words * 8 + words * 16 + 2 * (words + 1) * 4;
+    size_t cw = (gate_lds_limit() - gate_fixed_bytes(words)) / (ntp * 8);
+    if (cap > 0 && cw > (size_t)cap) cw = (size_t)cap;
+    return (int)(cw < words ? cw : words);
+}
+
+size_t gate_lds_bytes(int tile, int64_t nbK, int cap) {
+    const int MT = macro_dim(tile);
+    const size_t ntp = MT * MT < 8 ? 8 : MT * MT;
+    const size_t words = (size_t)((nbK + 63) / 64);
+    return ntp * (size_t)gate_chunk_words(tile, nbK, cap) * 8 + gate_fixed_bytes(words);
 }
 
 // k_gate may use all of a CU's LDS for the macro tile's bitmaps (its workgroups are short)
 hipError_t gate_init() {
     hipError_t e;
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)gate_lds_limit())) != hipSuccess) return e;
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<4>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)gate_lds_limit())) != hipSuccess) return e;
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gate<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)gate_lds_limit())) != hipSuccess) return e;
+    const void *gates[6] = {reinterpret_cast<const void *>(&k_gate<8, true>), reinterpret_cast<const void *>(&k_gate<8, false>),
+                            reinterpret_cast<const void *>(&k_gate<4, true>), reinterpret_cast<const void *>(&k_gate<4, false>),
+                            reinterpret_cast<const void *>(&k_gate<2, true>), reinterpret_cast<const void *>(&k_gate<2, false>)};
+    for (const void *f : gates)
+        if ((e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)gate_lds_limit())) != hipSuccess) return e;
     // k_order: its tables may take order_lds_limit() on top of a few static bytes
     return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_order), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)order_lds_limit());
 }
 
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
-                       float tau, int n_xcd, hipStream_t s) {
+                       float tau, int n_xcd, int chunk_cap, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nMacM = (int)((nbM + MT - 1) / MT), nMacN = (int)((nbN + MT - 1) / MT);
     const int n_macro = nMacM * nMacN;
-    const size_t lds = gate_lds_bytes(tile, nbK);
+    const size_t lds = gate_lds_bytes(tile, nbK, chunk_cap);
+    const int cw = gate_chunk_words(tile, nbK, chunk_cap);
+    const bool one = cw >= (int)((nbK + 63) / 64);
+#define SPAMM_GATE(MTV)                                                                                          \
+    if (one) k_gate<MTV, true><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw);      \
+    else k_gate<MTV, false><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw)
     switch (MT) {
-        case 8: k_gate<8><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
-        case 4: k_gate<4><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
-        case 2: k_gate<2><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau); break;
+        case 8: SPAMM_GATE(8); break;
+        case 4: SPAMM_GATE(4); break;
+        case 2: SPAMM_GATE(2); break;
         default: return hipErrorInvalidValue;
     }
+#undef SPAMM_GATE
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const int nSupM = (nMacM + SUPER_M - 1) / SUPER_M, nSupN = (nMacN + SUPER_N - 1) / SUPER_N;

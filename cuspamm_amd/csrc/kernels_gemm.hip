@@ -57,7 +57,10 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // every LDS read and serialise the staging ring); completion is awaited
 // explicitly with s_waitcnt vmcnt before the workgroup barrier.  M0 carries
 // the LDS address and is declared clobbered, so the compiler keeps nothing
-// live in it across a load.
+// live in it across a load.  Both scalar operands must come from scalar
+// instructions (as all callers' do): a VALU-written SGPR (v_readfirstlane)
+// read by a vector-memory instruction within five instructions is a hazard
+// the compiler does not see inside inline assembly.
 template <int IMM>
 __device__ __forceinline__ void dma_load(const unsigned char *sbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"

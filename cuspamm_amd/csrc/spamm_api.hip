@@ -60,6 +60,7 @@ struct spamm_ctx : Workspace {
     hipStream_t stream = nullptr;
     int last_hip = 0;
     int n_xcd = MAX_XCD;        // XCDs the GEMM schedule is built for (from the device's CU count)
+    int gate_chunk_cap = 0;     // developer knob SPAMM_GATE_CHUNK_WORDS: the gate's k chunk, 0 = what LDS holds
 
     Workspace parked;           // the workspace that is not live (see in_static)
     bool in_static = false;     // live workspace = carve-outs of the fixed device array
@@ -215,6 +216,10 @@ int spamm_create(spamm_ctx **out, int device) {
         const int n = atoi(env);
         if (n == 1 || n == 2 || n == 4 || n == 8) c->n_xcd = n;
     }
+    if (const char *env = getenv("SPAMM_GATE_CHUNK_WORDS")) {      // developer knob: gate's k chunk in 64-k words
+        const int n = atoi(env);
+        if (n > 0) c->gate_chunk_cap = n;
+    }
     int rc = set_device(c);
     if (rc == SPAMM_OK && hipStreamCreate(&c->own_stream) != hipSuccess) rc = SPAMM_EHIP;
     c->stream = c->own_stream;
@@ -364,7 +369,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
     int rc = set_device(c);
     if (rc) return rc;
     const Shape s = shape_of(c);
-    if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // K / tile beyond ~19 500 (tile 32)
+    if (gate_lds_bytes(c->tile, s.nbK) > gate_lds_limit()) return SPAMM_EINVAL;   // (defensive: the gate walks long K in chunks that fit)
     if (order_lds_bytes(c->tile, s.nbM, s.nbN) > order_lds_limit()) return SPAMM_EINVAL;   // more than 8192 super tiles of C
     const size_t nt = (size_t)s.nbM * s.nbN;
     if ((rc = ensure(c, c->counts, nt * 4))) return rc;
@@ -376,7 +381,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->sched, 2 * MAX_XCD * 4))) return rc;
     if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
-    HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->n_xcd, c->stream));
+    HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->n_xcd, c->gate_chunk_cap, c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[3], c->stream)); c->ev_gate = true; }
     c->tau = tau;
     c->have_gate = true;

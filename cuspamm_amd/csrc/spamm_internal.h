@@ -101,7 +101,7 @@ hipError_t launch_transpose_normmap(const float *nB, int64_t nbK, int64_t nbN, f
 hipError_t launch_fill_decay(float *X, int64_t rows, int64_t cols, const float *table,
                              uint64_t seed, int random, hipStream_t s);
 
-size_t gate_lds_bytes(int tile, int64_t nbK);
+size_t gate_lds_bytes(int tile, int64_t nbK, int chunk_cap = 0);   // chunk_cap > 0: at most that many 64-k words of bitmaps in LDS at a time
 inline size_t gate_lds_limit() { return 160 * 1024 - 64; }   // dynamic LDS of k_gate (a few static bytes aside)
 // k_order ranks the super tiles of C (4 x 8 macro tiles of 256 x 256) in one workgroup's LDS
 constexpr int LPT_MAX_SUPER = 2048;     // the greedy deal's table is laid out for at most this many super tiles,
@@ -123,7 +123,7 @@ inline size_t order_lds_bytes(int tile, int64_t nbM, int64_t nbN) {
 inline size_t order_lds_limit() { return 64 * 1024; }
 hipError_t gate_init();   // one-time kernel attribute set-up
 hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t nbN, int tile,
-                       float tau, int n_xcd, hipStream_t s);
+                       float tau, int n_xcd, int chunk_cap, hipStream_t s);
 // per-tile ascending k lists [n_tiles x nbK] from the gate's bitmaps (read-back only)
 hipError_t launch_klist(const uint64_t *mask, uint16_t *klist, int64_t n_tiles, int64_t nbK, hipStream_t s);
 

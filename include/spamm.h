@@ -143,8 +143,9 @@ SPAMM_API int spamm_normmap_f16(spamm_ctx *ctx, int role, const void *dXh, int64
  * ascending compacted k list of :315-325 is the bitmap's set bits in order;
  * spamm_get_klist materialises it).  Uses the norm maps left by stage 1 (or by
  * spamm_set_normmaps); SPAMM_ESTATE unless both are present for the same K and tile.
- * Shape limits (SPAMM_EINVAL): K / tile up to about 19 500 at tile 32 (a macro tile's bitmaps are
- * held in LDS; far more at tile 64 / 128), and at most 8192 super tiles of 1024 x 2048 elements of C. */
+ * Shape limit (SPAMM_EINVAL): at most 8192 super tiles of 1024 x 2048 elements of C.  K is not
+ * limited beyond the 65535 tiles per dimension: a macro tile's bitmaps are held in LDS, and where
+ * they do not fit (K / tile beyond about 19 500 at tile 32) the gate walks K in chunks. */
 SPAMM_API int spamm_gate(spamm_ctx *ctx, float tau);
 
 /* Stage 3 -- replaces the product loop of get_C_FP16_B32 (cuSpAMM.cu:336-391):

@@ -47,7 +47,8 @@ def test_random_shapes(orc, ctx):
                                         (288, 32, 2080, 32),
                                         (64, 576, 102400, 64),     # the reference's im2col shape (para.h:20-21)
                                         (32, 288000, 32, 32),      # 9000 k tiles: bitmaps beyond 64 KiB of LDS
-                                        (64, 65535 * 64, 64, 64)])  # the most k tiles the ABI takes
+                                        (64, 65535 * 64, 64, 64),  # the most k tiles the ABI takes
+                                        (32, 65535 * 32, 32, 32)])  # ... at tile 32: the gate walks k in four chunks
 def test_extreme_aspect_ratios(orc, ctx, M, K, N, tile):
     tab = orc.decay_table("exp", max(M, K, N), 0.002)
     A = orc.fill_decay(M, K, tab, 1)
@@ -76,6 +77,41 @@ def test_more_than_512_super_tiles_of_c(orc, ctx, M, n_sup_n, percents):
         B[:, cut:] = 0.0
         ref = _check(orc, ctx, A, B, tile, 1e-30)
         assert ref["kept"] == (M // tile) * (cut // tile)
+
+
+@pytest.mark.parametrize("chunk_words", [1, 3])
+def test_gate_in_small_k_chunks_gives_the_same_lists(orc, ctx, monkeypatch, chunk_words):
+    """A macro tile's bitmaps normally fit a CU's LDS whole; beyond ~19 500 k tiles (tile 32) the
+    gate walks k in chunks, twice.  Forcing chunks of 1 and 3 words (64 and 192 k tiles) sends
+    ordinary shapes down that path: mask, counts, kept total and C must not change by a bit."""
+    import torch
+    import cuspamm_amd as sp
+    monkeypatch.setenv("SPAMM_GATE_CHUNK_WORDS", str(chunk_words))     # read once, when the context is created
+    other = sp.SpammContext(0)
+    monkeypatch.delenv("SPAMM_GATE_CHUNK_WORDS")
+    try:
+        for (M, K, N), tile, lam, ratio in [((512, 8192, 768), 32, 0.004, 0.3), ((1024, 12800, 512), 64, 0.001, 0.5),
+                                            ((256, 33280, 384), 128, 0.0005, 0.4), ((320, 6432, 288), 32, 0.0, 1.0)]:
+            tab = orc.decay_table("exp", max(M, K, N), lam)
+            dA = torch.empty((M, K), dtype=torch.float32, device="cuda")
+            dB = torch.empty((K, N), dtype=torch.float32, device="cuda")
+            ctx.fill_decay(dA, tab, 1)
+            ctx.fill_decay(dB, tab, 2)
+            ctx.normmap_f32(1, dB, tile)
+            ctx.normmap_f32(0, dA, tile)
+            tau = 0.0 if ratio == 1.0 else ctx.tau_for_ratio(ratio)[0]
+            want = ctx.multiply(dA, dB, tile, tau)
+            mask, counts, kept = ctx.get_mask(), ctx.get_counts(), ctx.get_stats().kept_products
+            got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            other.multiply(dA, dB, tile, tau, C=got)
+            assert np.array_equal(other.get_mask(), mask)
+            assert np.array_equal(other.get_counts(), counts)
+            assert other.get_stats().kept_products == kept and 0 < kept
+            assert torch.equal(got, want)
+        tab = orc.decay_table("exp", 2048, 0.003)
+        _check(orc, other, orc.fill_decay(384, 2048, tab, 3), orc.fill_decay(2048, 320, tab, 4), 32, 0.05)
+    finally:
+        other.close()
 
 
 def test_scattered_sparsity_pattern(orc, ctx):
