@@ -1,0 +1,106 @@
+"""What the hand-written assembly in the kernels relies on, checked on the compiler's output.
+
+The compiler inserts the wait states gfx90a-and-later hardware needs between dependent
+instructions, but only around instructions it can see -- not around inline assembly:
+  * a vector-memory instruction must not read an SGPR that a VALU instruction (v_readfirstlane,
+    v_cmp with a scalar destination, ...) wrote within the five instructions before it;
+  * a VALU instruction must not read an SGPR that a VALU instruction wrote within the two before it.
+`dma_load` (kernels_gemm.hip: s_mov m0 / s_nop / global_load_lds) relies on its scalar operands
+coming from scalar instructions; `set_lane2` (kernels_gate.hip) carries its own s_nop.  This test
+compiles both files to gfx950 assembly (no GPU needed) and checks every assembly block."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "cuspamm_amd", "csrc")
+
+
+def _isa(src, tmp_path):
+    from cuspamm_amd import build
+    out = os.path.join(str(tmp_path), src.replace(".hip", ".s"))
+    cmd = [build.HIPCC] + [f for f in build.CFLAGS if f != "-Wall"] + ["-Wno-inline-asm", "-S", "--cuda-device-only",
+                                                                   os.path.join(CSRC, src), "-o", out]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    return open(out).read()
+
+
+def _sgprs(token):
+    """SGPR numbers named by one operand: s5 -> {5}, s[10:11] -> {10, 11}, vcc -> {'vcc'}."""
+    token = token.strip().rstrip(",")
+    m = re.fullmatch(r"s(\d+)", token)
+    if m:
+        return {int(m.group(1))}
+    m = re.fullmatch(r"s\[(\d+):(\d+)\]", token)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    if token in ("vcc", "vcc_lo", "vcc_hi"):
+        return {"vcc"}
+    return set()
+
+
+def _instructions(text):
+    """(mnemonic, operands, inside an inline-assembly block) per instruction line, in order."""
+    out, in_asm = [], False
+    for line in text.splitlines():
+        s = line.strip()
+        if s.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if s.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not s or s.startswith((";", ".", "/")) or s.endswith(":"):
+            continue
+        s = s.split(";")[0].strip()
+        if not s:
+            continue
+        parts = s.split(None, 1)
+        ops = [o.strip() for o in parts[1].split(",")] if len(parts) > 1 else []
+        out.append((parts[0], ops, in_asm))
+    return out
+
+
+def _valu_written_sgprs(mnemonic, ops):
+    """SGPRs a VALU instruction writes (scalar destination of a v_ instruction)."""
+    if not mnemonic.startswith("v_") or not ops:
+        return set()
+    written = _sgprs(ops[0])
+    if mnemonic.startswith(("v_cmp", "v_cmpx")) and mnemonic.endswith("_e32"):
+        written |= {"vcc"}
+    if re.match(r"v_(add|sub|subrev)_co_", mnemonic) and len(ops) > 1:
+        written |= _sgprs(ops[1])
+    return written
+
+
+def _wait_states(mnemonic, ops):
+    if mnemonic == "s_nop" and ops:
+        return int(ops[0], 0) + 1
+    return 1
+
+
+@pytest.mark.parametrize("src,reader,need", [("kernels_gemm.hip", "global_load_lds_dwordx4", 5),
+                                             ("kernels_gate.hip", "v_writelane_b32", 2)])
+def test_assembly_blocks_keep_their_distance_from_valu_written_sgprs(tmp_path, src, reader, need):
+    ins = _instructions(_isa(src, tmp_path))
+    checked = 0
+    for i, (mn, ops, in_asm) in enumerate(ins):
+        if not in_asm or mn != reader:
+            continue
+        checked += 1
+        read = set()
+        for o in ops:
+            read |= _sgprs(o.split()[0]) if o else set()
+        # walk back until `need` wait states lie between; any VALU write of a register we read is a hazard
+        states, j = 0, i - 1
+        while j >= 0 and states < need:
+            pmn, pops, _ = ins[j]
+            bad = _valu_written_sgprs(pmn, pops) & read
+            assert not bad, "%s: %s %s reads SGPR %s written %d wait states earlier by %s %s" % (
+                src, mn, ", ".join(ops), sorted(map(str, bad)), states, pmn, ", ".join(pops))
+            states += _wait_states(pmn, pops)
+            j -= 1
+    assert checked > 20, "no %s found inside assembly blocks of %s" % (reader, src)
