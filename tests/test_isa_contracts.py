@@ -7,7 +7,11 @@ instructions, but only around instructions it can see -- not around inline assem
   * a VALU instruction must not read an SGPR that a VALU instruction wrote within the two before it.
 `dma_load` (kernels_gemm.hip: s_mov m0 / s_nop / global_load_lds) relies on its scalar operands
 coming from scalar instructions; `set_lane2` (kernels_gate.hip) carries its own s_nop.  This test
-compiles both files to gfx950 assembly (no GPU needed) and checks every assembly block."""
+compiles both files to gfx950 assembly (no GPU needed) and checks every assembly block.
+
+The GEMM's k loops also wait for their global->LDS loads with hand-counted `s_waitcnt vmcnt(n)`:
+that count is right only while those loads are the only vector-memory instructions a wave issues
+between the first and the last of them, which the second test checks for every instantiation."""
 import os
 import re
 import subprocess
@@ -104,3 +108,19 @@ def test_assembly_blocks_keep_their_distance_from_valu_written_sgprs(tmp_path, s
             states += _wait_states(pmn, pops)
             j -= 1
     assert checked > 20, "no %s found inside assembly blocks of %s" % (reader, src)
+
+
+def test_gemm_k_loops_issue_no_other_vector_memory_instruction(tmp_path):
+    text = _isa("kernels_gemm.hip", tmp_path)
+    kernels = re.findall(r"^(_ZN5spamm6k_gemmILi\d+ELi\d+EEE\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
+    assert len(kernels) == 9          # tiles 32 / 64 / 128 x ring depths 3 / 4 / 5
+    for name, body in kernels:
+        mns = [mn for mn, _, _ in _instructions(body)]
+        dma = [i for i, mn in enumerate(mns) if mn == "global_load_lds_dwordx4"]
+        assert len(dma) >= 16, name
+        other = [mn for mn in mns[dma[0]:dma[-1] + 1]
+                 if mn.startswith(("global_", "flat_", "buffer_", "scratch_")) and mn != "global_load_lds_dwordx4"]
+        assert not other, "%s: %s between the first and the last global->LDS load" % (name, sorted(set(other)))
+        # and C is stored only after the loops have drained the ring
+        stores = [i for i, mn in enumerate(mns) if mn.startswith("global_store")]
+        assert stores and min(i for i in stores if i > dma[0]) > dma[-1], name
