@@ -221,7 +221,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         // the loops).  vmcnt counts completions in issue order, so "at most
         // LPW * (NBUF - 2) outstanding" means every load of the next stage
         // has landed.  Any other global load or store added inside the loops
-        // breaks this count: re-derive it.
+        // breaks this count: re-derive it (tests/test_isa_contracts.py checks
+        // the compiled assembly of every instantiation for it).
         auto sync_next = [&]() {
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(G::LPW * (NBUF - 2), 0));
             __syncthreads();
