@@ -45,7 +45,12 @@ WORKLOADS = {
     "cfg4_dense": (16384, 64, "none", 0.0, None, 0.0),
     "cfg5": (65536, 128, "exp", 0.003, 0.02, None),
     "cfg5_literal": (65536, 128, "exp", 0.05, 0.02, None),       # as written: 2 % unreachable
+    # the reference as checked out (para.h:1-14, cuSpAMM.cu:428-431): 2048^3, tile 32 (main.h:32), both operands
+    # 0.1 / (|i-j|^0.1 + 1) with no random factor (getDecayMatrixAlg, tool.cu:426-436), Norm = 1.548969, and
+    # fp16 inputs resident before the timed region (USINGHALF 1): the timed call is spamm_multiply_f16
+    "ref_default": (2048, 32, "ref_alg", 0.0, None, 1.548969),
 }
+FP16_INPUT_WORKLOADS = ("ref_default",)
 
 
 def measured_traffic(workload, profile_dir=PROFILE_DIR):
@@ -67,12 +72,30 @@ def measured_traffic(workload, profile_dir=PROFILE_DIR):
     return out
 
 
+def measured_trace_us(workload, profile_dir=PROFILE_DIR):
+    """Average kernel duration in microseconds by `rocprofv3 --kernel-trace --stats`, from the lines
+    `trace_us <workload> <kernel key> <microseconds>` of the committed summaries."""
+    out = {}
+    if not os.path.isdir(profile_dir):
+        return out
+    for name in sorted(os.listdir(profile_dir)):
+        if not name.endswith(".txt"):
+            continue
+        for line in open(os.path.join(profile_dir, name)):
+            f = line.split()
+            if len(f) == 4 and f[0] == "trace_us" and f[1] == workload:
+                out[f[2]] = float(f[3])
+    return out
+
+
 def decay_table(kind, n, lam):
     d = np.arange(n, dtype=np.float64)
     if kind == "exp":
         t = np.exp(-lam * d)
     elif kind == "alg":
         t = 1.0 / (1.0 + d) ** 2
+    elif kind == "ref_alg":                 # c / (d^v + 1), c = v = 0.1, evaluated as the reference does (float pow)
+        t = np.float32(0.1) / (np.power(d, np.float64(np.float32(0.1))).astype(np.float32) + np.float32(1))
     else:
         t = np.ones(n)
     return np.ascontiguousarray(t, dtype=np.float32)
@@ -138,6 +161,8 @@ def main():
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the timed multiplies (profiling runs): no ceiling probe, tau = 0 run, dense GEMM, "
                          "error report, literal config or CPU baseline")
+    ap.add_argument("--skip-variants", action="store_true",
+                    help="skip the fp16-input / REUSE_B / A_EQ_B / no-prune timings")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -162,7 +187,7 @@ def main():
         return
 
     if args.skip_extras:
-        args.no_cpu_baseline = args.skip_literal = args.skip_dense = True
+        args.no_cpu_baseline = args.skip_literal = args.skip_dense = args.skip_variants = True
     N, tile, kind, lam, ratio, tau = WORKLOADS[args.workload]
     nb = N // tile
     traffic = measured_traffic(args.workload)
@@ -170,9 +195,14 @@ def main():
     tab = decay_table(kind, N, lam)
     dA = torch.empty((N, N), dtype=torch.float32, device="cuda")
     dB = torch.empty((N, N), dtype=torch.float32, device="cuda")
-    ctx.fill_decay(dA, tab, 1)
-    ctx.fill_decay(dB, tab, 2)
+    det = kind == "ref_alg"                     # the reference's generators carry no random factor
+    ctx.fill_decay(dA, tab, 1, random=not det)
+    ctx.fill_decay(dB, tab, 2, random=not det)
     dC = torch.empty((N, N), dtype=torch.float32, device="cuda")
+    in16 = args.workload in FP16_INPUT_WORKLOADS
+    # operands of the timed call: the fp32 matrices, or (the reference's own timed region, para.h:1,
+    # cuSpAMM.cu:461-541) fp16 copies made before it
+    tA, tB = (dA.half(), dB.half()) if in16 else (dA, dB)
 
     if tau is None:
         # fixed before the timed region: exact order statistic over the norm products, on the device
@@ -186,24 +216,31 @@ def main():
     # tau is an argument of the call, so the A pass (second, as in the reference) can leave out
     # the fp16 copy of tiles that no product keeps: same C, mask and counts, fewer bytes written.
     prune = not args.no_prune
-    for _ in range(args.warmup):
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)
-    torch.cuda.synchronize()
+
+    def wall_ms(call, steps, warmup):
+        for _ in range(warmup):
+            call()
+        torch.cuda.synchronize()
+        t_0 = time.perf_counter()
+        for _ in range(steps):
+            call()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t_0) * 1e3 / steps
+
+    def event_ms(call, steps):
+        acc = np.zeros(5)
+        for _ in range(steps):
+            call()
+            s_ = ctx.get_stats()
+            acc += [s_.ms_normmap_b, s_.ms_normmap_a, s_.ms_gate, s_.ms_gemm, s_.ms_total]
+        return acc / steps, s_
+
     stage = np.zeros(5)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_step = wall * 1e3 / args.steps
+    ms_step = wall_ms(lambda: ctx.multiply(tA, tB, tile, tau, C=dC, prune=prune), args.steps, args.warmup)
     # per-kernel durations: HIP events recorded by the library on the stream the kernels run on;
     # re-run the same steps reading the events after each one (reading needs a sync, so it is
     # kept out of the wall-clock loop above)
-    for _ in range(args.steps):
-        ctx.multiply(dA, dB, tile, tau, C=dC, timing=True, prune=prune)
-        st = ctx.get_stats()
-        stage += [st.ms_normmap_b, st.ms_normmap_a, st.ms_gate, st.ms_gemm, st.ms_total]
-    stage /= args.steps
+    stage, st = event_ms(lambda: ctx.multiply(tA, tB, tile, tau, C=dC, timing=True, prune=prune), args.steps)
     # bytes the A pass writes: tile (i, k) is copied iff fl32(nA[i,k] * max_j nB[k,j]) >= tau
     nA_h, nB_h = ctx.get_normmap(sp.ROLE_A), ctx.get_normmap(sp.ROLE_B)
     # and the B pass every tile of non-zero norm
@@ -215,9 +252,20 @@ def main():
     flops = kept * 2.0 * tile ** 3
     value = flops / (ms_step * 1e-3) / 1e12
     gemm_tflops = flops / (stage[3] * 1e-3) / 1e12
-    nm_bytes = 4.0 * N * N + 2.0 * N * N + 4.0 * nb * nb               # per matrix, every tile written
-    nm_bytes_a = 4.0 * N * N + 2.0 * tile * tile * a_written + 4.0 * nb * nb
-    nm_bytes_b = 4.0 * N * N + 2.0 * tile * tile * b_written + 8.0 * nb * nb
+    in_b = 2.0 if in16 else 4.0                                         # bytes per input element
+    nm_bytes = in_b * N * N + 2.0 * N * N + 4.0 * nb * nb               # per matrix, every tile written
+    nm_bytes_a = in_b * N * N + 2.0 * tile * tile * a_written + 4.0 * nb * nb
+    nm_bytes_b = in_b * N * N + 2.0 * tile * tile * b_written + 8.0 * nb * nb
+    # operand bytes the GEMM must read at least once: the distinct fp16 tiles A(i,k) / B(k,j) that some
+    # kept product uses (from the gate's own bitmap), plus C written once
+    gm = ctx.get_mask()                                                 # [nbM, nbN, words] uint64, bit k
+    a_need = np.bitwise_or.reduce(gm, axis=1)                           # [nbM, words]: k tiles row i needs
+    b_need = np.bitwise_or.reduce(gm, axis=0)                           # [nbN, words]
+    a_tiles_read = int(np.unpackbits(a_need.view(np.uint8)).sum())
+    b_tiles_read = int(np.unpackbits(b_need.view(np.uint8)).sum())
+    del gm
+    gemm_alg_bytes = 4.0 * N * N + 2.0 * tile * tile * (a_tiles_read + b_tiles_read)
+    trace_us = measured_trace_us(args.workload)
     nm_gbs = nm_bytes_b / (stage[0] * 1e-3) / 1e9                      # the B pass
 
     out = {
@@ -239,7 +287,7 @@ def main():
             "name": args.workload, "N": N, "tile": tile, "tau": tau, "target_kept_fraction": ratio,
             "kept_products": kept, "total_products": total,
             "kept_fraction": round(kept / total, 5),
-            "prune": prune,
+            "prune": prune, "inputs": "fp16" if in16 else "fp32",
         },
         "stage_ms": {"normmap_b": round(stage[0], 4), "normmap_a": round(stage[1], 4), "gate": round(stage[2], 4),
                      "gemm": round(stage[3], 4), "sum_events": round(stage[4], 4)},
@@ -252,6 +300,14 @@ def main():
             "frac": round(gemm_tflops / PEAK_FP16_TFLOPS, 4),
             "traffic": traffic.get("k_gemm"),
             "flops_per_launch": flops, "avg_launch_ms": round(stage[3], 4),
+            "frac_basis": "HIP events recorded by the library around the kernel on its stream, this run",
+            "frac_by_kernel_trace": (round(flops / (trace_us["k_gemm"] * 1e-6) / 1e12 / PEAK_FP16_TFLOPS, 4)
+                                     if "k_gemm" in trace_us else None),
+            "kernel_trace_avg_launch_ms": round(trace_us["k_gemm"] * 1e-3, 4) if "k_gemm" in trace_us else None,
+            "kernel_trace_basis": "rocprofv3 --kernel-trace average of the committed profiles/ summary (another run, another box)",
+            "algorithmic_bytes_per_launch": gemm_alg_bytes,
+            "algorithmic_operand_tiles": {"a": a_tiles_read, "b": b_tiles_read, "tile_bytes": 2 * tile * tile},
+            "traffic_over_algorithmic": (round(traffic["k_gemm"] / gemm_alg_bytes, 3) if "k_gemm" in traffic else None),
         },
         "roofline_normmap": {
             "kernel": "k_normmap<%d, B role> (fp32->fp16 + tile norms)" % tile, "bound": "hbm",
@@ -259,21 +315,81 @@ def main():
             "frac": round(nm_gbs / PEAK_HBM_GBS, 4),
             "traffic": traffic.get("k_normmap_b" if pruned else "k_normmap_b_unpruned"),
             "bytes_per_launch": nm_bytes_b, "avg_launch_ms": round(stage[0], 4),
+            "frac_basis": "HIP events: the first stage's interval includes the gap before its kernel starts",
+            "frac_by_kernel_trace": (round(nm_bytes_b / (trace_us["k_normmap_b"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)
+                                     if "k_normmap_b" in trace_us and pruned else None),
+            "kernel_trace_avg_launch_ms": round(trace_us["k_normmap_b"] * 1e-3, 4) if "k_normmap_b" in trace_us else None,
             "tiles_written": b_written, "tiles": a_tiles, "bytes_per_launch_all_tiles": nm_bytes,
             "a_pass": {"tiles_written": a_written, "tiles": a_tiles, "bytes_per_launch": nm_bytes_a,
                        "avg_launch_ms": round(stage[1], 4),
                        "achieved": round(nm_bytes_a / (stage[1] * 1e-3) / 1e9, 1),
+                       "frac": round(nm_bytes_a / (stage[1] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                       "frac_basis": "HIP events: the interval also covers k_rowmax (a few microseconds)",
+                       "frac_by_kernel_trace": (round(nm_bytes_a / (trace_us["k_normmap_a"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)
+                                                if "k_normmap_a" in trace_us and pruned else None),
                        "traffic": traffic.get("k_normmap_a" if pruned else "k_normmap_a_unpruned")},
         },
     }
+
+    # The same multiply under the library's other calling conventions, each timed like the headline
+    # (wall clock over whole calls, then per-stage events), outside the headline's timed loop.
+    if not args.skip_variants:
+        vsteps, vwarm = max(5, args.steps // 2), max(2, args.warmup // 2)
+        variants = {}
+
+        def variant(name, what, call_plain, call_timed, in_bytes_elem=None, written=None):
+            ms = wall_ms(call_plain, vsteps, vwarm)
+            sg, s_ = event_ms(call_timed, vsteps)
+            fl = s_.kept_products * 2.0 * tile ** 3
+            v = {"what": what, "ms_per_step": round(ms, 4), "value_tflops": round(fl / (ms * 1e-3) / 1e12, 2),
+                 "kept_products": int(s_.kept_products),
+                 "stage_ms": {"normmap_b": round(sg[0], 4), "normmap_a": round(sg[1], 4), "gate": round(sg[2], 4),
+                              "gemm": round(sg[3], 4)}}
+            if in_bytes_elem is not None:
+                bw, aw = written
+                bb = in_bytes_elem * N * N + 2.0 * tile * tile * bw + 8.0 * nb * nb
+                ba = in_bytes_elem * N * N + 2.0 * tile * tile * aw + 4.0 * nb * nb
+                v["normmap_b_pass"] = {"bytes_per_launch": bb, "GBps": round(bb / (sg[0] * 1e-3) / 1e9, 1),
+                                       "frac_of_hbm_peak": round(bb / (sg[0] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+                v["normmap_a_pass"] = {"bytes_per_launch": ba, "GBps": round(ba / (sg[1] * 1e-3) / 1e9, 1),
+                                       "frac_of_hbm_peak": round(ba / (sg[1] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+            variants[name] = v
+
+        if prune:
+            variant("no_prune", "the timed call without SPAMM_FLAG_PRUNE: both passes write every fp16 tile",
+                    lambda: ctx.multiply(tA, tB, tile, tau, C=dC),
+                    lambda: ctx.multiply(tA, tB, tile, tau, C=dC, timing=True), in_b, (a_tiles, a_tiles))
+        if not in16:
+            hA, hB = dA.half(), dB.half()
+            variant("fp16_inputs", "spamm_multiply_f16 on fp16 copies made before the timed region (the reference's "
+                    "own timed region: para.h:1, cuSpAMM.cu:461-541); passes read 2 bytes per element",
+                    lambda: ctx.multiply(hA, hB, tile, tau, C=dC, prune=prune),
+                    lambda: ctx.multiply(hA, hB, tile, tau, C=dC, timing=True, prune=prune), 2.0, (b_written, a_written))
+            del hA, hB
+        # one B against many A: B's fp16 copy and norm map stay resident (A's pass, gate, GEMM remain)
+        ctx.multiply(tA, tB, tile, tau, C=dC, prune=prune)
+        variant("reuse_b", "SPAMM_FLAG_REUSE_B: B's fp16 copy and norm map kept from the previous call",
+                lambda: ctx.multiply(tA, tB, tile, tau, C=dC, prune=prune, reuse_b=True),
+                lambda: ctx.multiply(tA, tB, tile, tau, C=dC, timing=True, prune=prune, reuse_b=True))
+        # A = B (BASELINE's first configuration, matrix powers): one read feeds both operand roles; the product
+        # is A*A, so its kept count is its own
+        variant("a_eq_b", "SPAMM_FLAG_A_EQ_B on A*A: one pass reads the matrix once and writes both packed copies "
+                "(reported as normmap_b); beside it the same product as two passes",
+                lambda: ctx.multiply(tA, tA, tile, tau, C=dC, prune=prune, a_eq_b=True),
+                lambda: ctx.multiply(tA, tA, tile, tau, C=dC, timing=True, prune=prune, a_eq_b=True))
+        variants["a_eq_b"]["two_pass_ms_per_step"] = round(
+            wall_ms(lambda: ctx.multiply(tA, tA, tile, tau, C=dC, prune=prune), vsteps, vwarm), 4)
+        out["variants"] = variants
+        out["no_prune_ms_per_step"] = variants["no_prune"]["ms_per_step"] if "no_prune" in variants else round(ms_step, 4)
 
     # what the matrix pipeline sustains on this box with nothing but MFMAs: with random operands
     # the clock settles well below the datasheet's (power management), so this, not the datasheet
     # peak, is what a GEMM on real data can approach; and a dense fp16 GEMM of the same size by the
     # vendor library (the analogue of the reference's cuBLAS comparison, tool.cu:153-226)
     if not args.skip_extras:
-        tf_rand, ghz_rand = ctx.mfma_ceiling(True)
-        tf_zero, ghz_zero = ctx.mfma_ceiling(False)
+        from cuspamm_amd import dev as spdev
+        tf_rand, ghz_rand = spdev.mfma_ceiling(0, True)
+        tf_zero, ghz_zero = spdev.mfma_ceiling(0, False)
         out["mfma_ceiling"] = {
             "random_operands_tflops": round(tf_rand, 1), "random_operands_clock_ghz": round(ghz_rand, 3),
             "zero_operands_tflops": round(tf_zero, 1), "zero_operands_clock_ghz": round(ghz_zero, 3),
@@ -316,7 +432,7 @@ def main():
     # error against an exact fp64 dense product of the same fp16 operands, whole matrix, next to
     # the tau-derived bound (both formed on the device, outside the timed region)
     if N <= 16384 and not args.skip_extras:
-        ctx.multiply(dA, dB, tile, tau, C=dC)
+        ctx.multiply(tA, tB, tile, tau, C=dC)
         e64, d64, c64 = ctx.error_vs_dense(dC)
         bound = ctx.dropped_bound(tau)
         # fp32 accumulation of K terms leaves ~eps32 * sqrt(K) relative noise on the kept part even
@@ -399,8 +515,8 @@ def main():
         A, B = dA.cpu().numpy(), dB.cpu().numpy()
         same_c = None
         if prune:
-            plain = ctx.multiply(dA, dB, tile, tau).clone()
-        ctx.multiply(dA, dB, tile, tau, C=dC, prune=prune)      # the call that was timed
+            plain = ctx.multiply(tA, tB, tile, tau).clone()
+        ctx.multiply(tA, tB, tile, tau, C=dC, prune=prune)      # the call that was timed
         if prune:
             same_c = bool(torch.equal(plain, dC))
             del plain

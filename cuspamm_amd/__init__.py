@@ -14,6 +14,9 @@ from .api import (  # noqa: F401
     FLAG_REUSE_B,
     FLAG_PRUNE,
     NOALLOC_WORKSPACE_BYTES,
+    OPT_NUM_XCD,
+    OPT_GATE_CHUNK_WORDS,
+    OPT_GEMM_RING,
     SpammContext,
     SpammError,
     SpammParams,

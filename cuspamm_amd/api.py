@@ -19,6 +19,8 @@ FLAG_REUSE_A = 4
 FLAG_REUSE_B = 8
 FLAG_PRUNE = 16
 
+OPT_NUM_XCD, OPT_GATE_CHUNK_WORDS, OPT_GEMM_RING = 1, 2, 3
+
 OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV, ELIMIT = 0, -1, -2, -3, -4, -5, -6
 NOALLOC_WORKSPACE_BYTES = 40 << 20
 
@@ -75,8 +77,8 @@ def load_library():
     L.spamm_multiply_f16.argtypes = [vp, ctypes.POINTER(SpammParams), vp, vp, vp]
     L.spamm_error_vs_dense_f64.argtypes = [vp, vp, i64, i64, ctypes.POINTER(ctypes.c_double)]
     L.spamm_dropped_bound.argtypes = [vp, f32, ctypes.POINTER(ctypes.c_double)]
-    L.spamm_mfma_ceiling.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
-                                     ctypes.POINTER(ctypes.c_double)]
+    L.spamm_dropped_bound_tiles.argtypes = [vp, f32, vp]
+    L.spamm_set_option.argtypes = [vp, ctypes.c_int, ctypes.c_int]
     L.spamm_load_csv_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
     L.spamm_load_mtx_f32.argtypes = [ctypes.c_char_p, i64, i64, i64, vp]
     L.spamm_gate.argtypes = [vp, f32]
@@ -127,6 +129,15 @@ def _devptr(t, dtype_name):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _check_out(A, B, C, M, N):
+    """The GEMM writes M x N floats through C's pointer: refuse anything smaller or elsewhere before
+    a kernel is launched (an out-of-bounds store is a device fault, not an error code)."""
+    if getattr(C, "dim", lambda: 0)() != 2 or tuple(C.shape) != (M, N):
+        raise ValueError("C must have shape (%d, %d), got %s" % (M, N, tuple(getattr(C, "shape", ()))))
+    if B.device != A.device or C.device != A.device:
+        raise ValueError("A, B and C must be on the same device")
+
+
 class SpammContext:
     """One device + one stream + reusable workspaces (spamm_ctx)."""
 
@@ -162,6 +173,9 @@ class SpammContext:
         _check(self._lib.spamm_set_stream(self._h, ctypes.c_void_p(raw_stream or 0)),
                "spamm_set_stream")
 
+    def set_option(self, option, value):
+        _check(self._lib.spamm_set_option(self._h, int(option), int(value)), "spamm_set_option")
+
     def synchronize(self):
         _check(self._lib.spamm_synchronize(self._h), "spamm_synchronize")
 
@@ -186,6 +200,7 @@ class SpammContext:
             raise TypeError("A and B must have the same dtype")
         if C is None:
             C = torch.empty((M, N), dtype=torch.float32, device=A.device)
+        _check_out(A, B, C, M, N)
         flags = ((FLAG_TIMING if timing else 0) | (FLAG_REUSE_A if reuse_a else 0) |
                  (FLAG_REUSE_B if reuse_b else 0) | (FLAG_A_EQ_B if a_eq_b else 0) |
                  (FLAG_PRUNE if prune else 0))
@@ -204,10 +219,13 @@ class SpammContext:
     def multiply_noalloc(self, A, B, tile, tau, C, timing=False, a_eq_b=False, prune=False):
         """spamm_multiply_noalloc: the same multiply in the library's fixed device workspace (fp32 inputs,
         caller-provided C, no device allocation inside the call; SpammError ELIMIT beyond the workspace)."""
+        if getattr(A, "dim", lambda: 0)() != 2 or getattr(B, "dim", lambda: 0)() != 2:
+            raise ValueError("A and B must be matrices")
         M, K = A.shape
         K2, N = B.shape
         if K != K2:
             raise ValueError("inner dimensions differ")
+        _check_out(A, B, C, M, N)
         flags = (FLAG_TIMING if timing else 0) | (FLAG_A_EQ_B if a_eq_b else 0) | (FLAG_PRUNE if prune else 0)
         p = SpammParams(M, K, N, int(tile), float(tau), flags, 0)
         _check(self._lib.spamm_multiply_noalloc(self._h, ctypes.byref(p), _devptr(A, "float32"),
@@ -254,12 +272,12 @@ class SpammContext:
                "spamm_error_vs_dense_f64")
         return out[0], out[1], out[2]
 
-    def mfma_ceiling(self, random_operands=True, iters=20000):
-        """(TFLOP/s, GHz) of a pure MFMA issue loop on every CU; a measurement aid."""
-        tf, ghz = ctypes.c_double(0), ctypes.c_double(0)
-        _check(self._lib.spamm_mfma_ceiling(self._h, int(bool(random_operands)), int(iters), ctypes.byref(tf),
-                                            ctypes.byref(ghz)), "spamm_mfma_ceiling")
-        return float(tf.value), float(ghz.value)
+    def dropped_bound_tiles(self, tau):
+        """Per output tile: sum over dropped k of nA[i,k]*nB[k,j] (float64 [nbM, nbN])."""
+        nbM, nbK, nbN = self._shape[:3]
+        out = np.empty((nbM, nbN), dtype=np.float64)
+        _check(self._lib.spamm_dropped_bound_tiles(self._h, float(tau), out.ctypes.data), "spamm_dropped_bound_tiles")
+        return out
 
     def dropped_bound(self, tau):
         out = ctypes.c_double(0)

@@ -11,6 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libspamm_gfx950.so")
+DEV_LIB_PATH = os.path.join(HERE, "libspamm_dev_gfx950.so")   # measurement aids (csrc/dev_probe.hip), not the engine
 MAIN_PATH = os.path.join(HERE, "spamm_main")     # the reference's main() on top of the C ABI (csrc/spamm_main.cpp)
 
 SOURCES = ["kernels_normmap.hip", "kernels_gate.hip", "kernels_gemm.hip", "kernels_tau.hip", "kernels_tools.hip",
@@ -86,6 +87,7 @@ def build_library(verbose=False):
     with ThreadPoolExecutor(max_workers=4) as ex:
         logs = list(ex.map(compile_one, zip(SOURCES, objs)))
     logs.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs))
+    logs.append(_run([HIPCC] + CFLAGS + ["-shared", os.path.join(CSRC, "dev_probe.hip"), "-o", DEV_LIB_PATH]))
     logs.append(_run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wall", os.path.join(CSRC, "spamm_main.cpp"), "-o", MAIN_PATH,
                       "-L" + HERE, "-lspamm_gfx950", "-Wl,-rpath,$ORIGIN"]))
     if verbose:

@@ -401,8 +401,6 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     }
 }
 
-static int g_nbuf = 4;
-
 template <int B, int NBUF>
 static hipError_t set_lds_attr() {
     return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, NBUF>),
@@ -410,8 +408,6 @@ static hipError_t set_lds_attr() {
 }
 
 hipError_t gemm_init() {
-    const char *env = getenv("SPAMM_GEMM_NBUF");     // developer tuning knob: depth of the LDS ring
-    if (env && (env[0] == '3' || env[0] == '4' || env[0] == '5')) g_nbuf = env[0] - '0';
     hipError_t e;
     if ((e = set_lds_attr<32, 3>()) != hipSuccess) return e;
     if ((e = set_lds_attr<32, 4>()) != hipSuccess) return e;
@@ -443,7 +439,7 @@ static void launch_tile(int nbuf, unsigned grid, int n_xcd, const unsigned char 
 }
 
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, hipStream_t s) {
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
@@ -453,9 +449,9 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
     switch (tile) {
-        case 32: launch_tile<32>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 64: launch_tile<64>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 128: launch_tile<128>(g_nbuf, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 32: launch_tile<32>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 64: launch_tile<64>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 128: launch_tile<128>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -105,23 +105,38 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
     const int64_t eoff = (I * B) * ld + col0 + cl;
 
     f32x4 v[NGW][8];
+    if (IN16) {
+        // every lane loads unconditionally (a lane beyond the last column reads the strip's first
+        // column instead and zeroes the values afterwards): with the loads inside a branch the
+        // compiler waits for each one before it issues the next
+        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+        const _Float16 *src = static_cast<const _Float16 *>(Xv) + (valid ? eoff : (I * B) * ld + col0);
+        half4v hv[NGW][8];
 #pragma unroll
-    for (int i = 0; i < NGW; i++)
+        for (int i = 0; i < NGW; i++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int r = 8 * (g0 + GSTEP * i) + j;
-            if (!valid) {
-                v[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            } else if (IN16) {
-                typedef _Float16 half4v __attribute__((ext_vector_type(4)));
-                const half4v hv = __builtin_nontemporal_load(
-                    reinterpret_cast<const half4v *>(static_cast<const _Float16 *>(Xv) + eoff + (int64_t)r * ld));
-                v[i][j] = f32x4{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
-            } else {
-                v[i][j] = __builtin_nontemporal_load(
-                    reinterpret_cast<const f32x4 *>(static_cast<const float *>(Xv) + eoff + (int64_t)r * ld));
+            for (int j = 0; j < 8; j++)
+                hv[i][j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const half4v *>(src + (int64_t)(8 * (g0 + GSTEP * i) + j) * ld));
+#pragma unroll
+        for (int i = 0; i < NGW; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                v[i][j] = valid ? f32x4{(float)hv[i][j].x, (float)hv[i][j].y, (float)hv[i][j].z, (float)hv[i][j].w}
+                                : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    } else {
+#pragma unroll
+        for (int i = 0; i < NGW; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int r = 8 * (g0 + GSTEP * i) + j;
+                if (!valid)
+                    v[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                else
+                    v[i][j] = __builtin_nontemporal_load(
+                        reinterpret_cast<const f32x4 *>(static_cast<const float *>(Xv) + eoff + (int64_t)r * ld));
             }
-        }
+    }
 
     // ROLE 2 = the same matrix is both operands (A = B): one read of X, both packed layouts and
     // both norm maps (A role first -> packed/nm, then B role -> packed2/nm2/nmT), LDS reused.

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void k_error_dense(const _Float16 *__restrict_
 
 __global__ __launch_bounds__(256) void k_dropped_bound(const float *__restrict__ nA, const float *__restrict__ nBt,
                                                        int nbM, int nbK, int nbN, float tau,
-                                                       double *__restrict__ out) {
+                                                       double *__restrict__ out, double *__restrict__ per_tile) {
     // one wave per output tile
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -91,7 +91,10 @@ __global__ __launch_bounds__(256) void k_dropped_bound(const float *__restrict__
         if (!(p >= tau)) s += (double)a * (double)b;
     }
     for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
-    if (lane == 0) atomicAdd(out, s * s);
+    if (lane == 0) {
+        atomicAdd(out, s * s);
+        if (per_tile) per_tile[t] = s;
+    }
 }
 
 __global__ void k_clear_f64(double *p, int n) {
@@ -110,54 +113,10 @@ hipError_t launch_error_vs_dense(const void *packedA, const void *packedB, int64
 }
 
 hipError_t launch_dropped_bound(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
-                                float tau, double *out1, hipStream_t s) {
+                                float tau, double *out1, double *per_tile, hipStream_t s) {
     k_clear_f64<<<1, 64, 0, s>>>(out1, 1);
     const int64_t nt = nbM * nbN;
-    k_dropped_bound<<<(unsigned)((nt + 3) / 4), 256, 0, s>>>(nA, nBt, (int)nbM, (int)nbK, (int)nbN, tau, out1);
-    return hipGetLastError();
-}
-
-// ---- matrix-pipeline ceiling: a grid of one workgroup per CU (4 waves, one per SIMD) that issues
-// nothing but independent 32x32x16 fp16 MFMAs on 16 accumulator blocks per wave.  On this part the
-// sustained clock under MFMA load depends on the operand values (power management), so the rate
-// measured here with operands like the workload's is the ceiling a GEMM can reach, below the
-// datasheet peak.  trace[2 b] = 100 MHz wall ticks, trace[2 b + 1] = shader clocks of workgroup b.
-typedef _Float16 ceil_half8 __attribute__((ext_vector_type(8)));
-typedef float ceil_f32x16 __attribute__((ext_vector_type(16)));
-__global__ __launch_bounds__(256) void k_mfma_ceiling(const ceil_half8 *__restrict__ in, float *__restrict__ out,
-                                                      unsigned long long *__restrict__ trace, int iters) {
-    ceil_half8 a[4], b[4];
-    for (int i = 0; i < 4; i++) {
-        a[i] = in[(i * 256 + threadIdx.x) % 2048];
-        b[i] = in[((i + 4) * 256 + threadIdx.x) % 2048];
-    }
-    ceil_f32x16 acc[4][4];
-    for (int r = 0; r < 4; r++)
-        for (int c = 0; c < 4; c++)
-            for (int i = 0; i < 16; i++) acc[r][c][i] = 0.0f;
-    const unsigned long long w0 = wall_clock64(), c0 = clock64();
-    for (int it = 0; it < iters; it++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-                acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[r], b[c], acc[r][c], 0, 0, 0);
-    }
-    const unsigned long long c1 = clock64(), w1 = wall_clock64();
-    float s = 0.0f;
-    for (int r = 0; r < 4; r++)
-        for (int c = 0; c < 4; c++)
-            for (int i = 0; i < 16; i++) s += acc[r][c][i];
-    out[blockIdx.x * 256 + threadIdx.x] = s;
-    if (threadIdx.x == 0) {
-        trace[blockIdx.x * 2] = w1 - w0;
-        trace[blockIdx.x * 2 + 1] = c1 - c0;
-    }
-}
-
-hipError_t launch_mfma_ceiling(const void *in2048x16B, float *out, unsigned long long *trace, int n_wg, int iters,
-                               hipStream_t s) {
-    k_mfma_ceiling<<<n_wg, 256, 0, s>>>((const ceil_half8 *)in2048x16B, out, trace, iters);
+    k_dropped_bound<<<(unsigned)((nt + 3) / 4), 256, 0, s>>>(nA, nBt, (int)nbM, (int)nbK, (int)nbN, tau, out1, per_tile);
     return hipGetLastError();
 }
 

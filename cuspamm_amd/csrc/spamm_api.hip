@@ -4,6 +4,7 @@
 #include "../../include/spamm.h"
 
 #include <math.h>
+#include <atomic>
 #include <new>
 #include <utility>
 #include <stdio.h>
@@ -20,6 +21,12 @@ using namespace spamm;
 // handle for hipGetSymbolAddress: the device address is looked up once per context (= per device)
 // in spamm_create and everything below uses that pointer.
 static __device__ __align__(256) unsigned char scratch[SPAMM_NOALLOC_WORKSPACE_BYTES];
+
+// Every spamm_multiply_noalloc on a device overwrites that device's array, whichever context makes
+// the call: a per-device generation number, bumped by each such call, tells a context whether what
+// it left there is still its own (see static_stale).
+static constexpr int MAX_DEVICES = 64;
+static std::atomic<uint64_t> g_static_gen[MAX_DEVICES];
 
 namespace {
 
@@ -60,7 +67,9 @@ struct spamm_ctx : Workspace {
     hipStream_t stream = nullptr;
     int last_hip = 0;
     int n_xcd = MAX_XCD;        // XCDs the GEMM schedule is built for (from the device's CU count)
-    int gate_chunk_cap = 0;     // developer knob SPAMM_GATE_CHUNK_WORDS: the gate's k chunk, 0 = what LDS holds
+    int gate_chunk_cap = 0;     // SPAMM_OPT_GATE_CHUNK_WORDS: the gate's k chunk, 0 = what LDS holds
+    int gemm_ring = 4;          // SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's staging ring
+    uint64_t static_gen = 0;    // generation of the fixed array this context's noalloc results belong to
 
     Workspace parked;           // the workspace that is not live (see in_static)
     bool in_static = false;     // live workspace = carve-outs of the fixed device array
@@ -169,6 +178,12 @@ void leave_static(spamm_ctx *c) {
     c->in_static = false;
 }
 
+// The live workspace is the fixed array and another spamm_multiply_noalloc on this device (from
+// any context) has overwritten it since: nothing this context left there can be read or consumed.
+bool static_stale(const spamm_ctx *c) {
+    return c->in_static && c->static_gen != g_static_gen[c->device].load(std::memory_order_acquire);
+}
+
 int copy_out(spamm_ctx *c, const void *dev, void *host, size_t bytes) {
     HIPCHK(c, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
@@ -202,7 +217,7 @@ int spamm_create(spamm_ctx **out, int device) {
         (void)hipGetLastError();
         return SPAMM_ENODEV;
     }
-    if (device < 0 || device >= ndev) return SPAMM_EINVAL;
+    if (device < 0 || device >= ndev || device >= MAX_DEVICES) return SPAMM_EINVAL;
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) != hipSuccess) return SPAMM_ENODEV;
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return SPAMM_ENODEV;
@@ -212,14 +227,6 @@ int spamm_create(spamm_ctx **out, int device) {
     // the schedule groups workgroups by XCD (32 CUs sharing an L2): 256 CUs = 8 XCDs; a partitioned
     // device shows 128 / 64 / 32 CUs; any other CU count gets one flat sequence
     c->n_xcd = xcds_for_cu_count(prop.multiProcessorCount);
-    if (const char *env = getenv("SPAMM_NUM_XCD")) {      // developer knob: 1, 2, 4 or 8
-        const int n = atoi(env);
-        if (n == 1 || n == 2 || n == 4 || n == 8) c->n_xcd = n;
-    }
-    if (const char *env = getenv("SPAMM_GATE_CHUNK_WORDS")) {      // developer knob: gate's k chunk in 64-k words
-        const int n = atoi(env);
-        if (n > 0) c->gate_chunk_cap = n;
-    }
     int rc = set_device(c);
     if (rc == SPAMM_OK && hipStreamCreate(&c->own_stream) != hipSuccess) rc = SPAMM_EHIP;
     c->stream = c->own_stream;
@@ -260,6 +267,33 @@ int spamm_set_stream(spamm_ctx *c, void *hip_stream) {
     if (!c) return SPAMM_EINVAL;
     c->stream = hip_stream ? (hipStream_t)hip_stream : c->own_stream;
     return SPAMM_OK;
+}
+
+int spamm_set_option(spamm_ctx *c, int option, int value) {
+    if (!c) return SPAMM_EINVAL;
+    switch (option) {
+        case SPAMM_OPT_NUM_XCD:
+            if (value == 0) {
+                hipDeviceProp_t prop;
+                if (hipGetDeviceProperties(&prop, c->device) != hipSuccess) return SPAMM_EHIP;
+                value = xcds_for_cu_count(prop.multiProcessorCount);
+            }
+            if (value != 1 && value != 2 && value != 4 && value != 8) return SPAMM_EINVAL;
+            c->n_xcd = value;
+            c->have_gate = false;          // the schedule was built for the old count
+            return SPAMM_OK;
+        case SPAMM_OPT_GATE_CHUNK_WORDS:
+            if (value < 0) return SPAMM_EINVAL;
+            c->gate_chunk_cap = value;
+            return SPAMM_OK;
+        case SPAMM_OPT_GEMM_RING:
+            if (value == 0) value = 4;
+            if (value < 3 || value > 5) return SPAMM_EINVAL;
+            c->gemm_ring = value;
+            return SPAMM_OK;
+        default:
+            return SPAMM_EINVAL;
+    }
 }
 
 int spamm_last_hip_error(spamm_ctx *c) { return c ? c->last_hip : 0; }
@@ -364,6 +398,7 @@ int spamm_set_normmaps(spamm_ctx *c, const float *nA, const float *nB, int64_t n
 
 int spamm_gate(spamm_ctx *c, float tau) {
     if (!c) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     if (tau != tau) return SPAMM_EINVAL;   // NaN
     int rc = set_device(c);
@@ -390,6 +425,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
 
 int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (!c || !dC) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->have_a || !c->have_b || !c->have_gate) return SPAMM_ESTATE;
     if (c->a_pruned && !(c->tau >= c->a_pruned_tau)) return SPAMM_ESTATE;   // A's copy lacks tiles this tau keeps
     if (c->b_pruned && !(c->tau > 0.0f)) return SPAMM_ESTATE;               // B's copy lacks its zero tiles
@@ -397,7 +433,7 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
     HIPCHK(c, launch_gemm(c->packedA.p, c->packedB.p, gate_buffers(c), c->M, c->K, c->N, c->tile, dC,
-                          c->n_xcd, c->stream));
+                          c->n_xcd, c->gemm_ring, c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[4], c->stream)); c->ev_gemm = true; }
     return SPAMM_OK;
 }
@@ -530,6 +566,7 @@ int spamm_multiply_noalloc(spamm_ctx *c, const spamm_params *p, const float *dA,
         c->in_static = true;
     }
     reset_shape(c, p->tile);           // the carve-outs move with the shape, and other contexts share the array
+    c->static_gen = g_static_gen[c->device].fetch_add(1, std::memory_order_acq_rel) + 1;
     (void)carve_static(*c, p, c->static_ptr);
     c->no_alloc = true;
     const int rc = multiply_any(c, p, dA, dB, false, dC);
@@ -547,6 +584,7 @@ int spamm_multiply_f16(spamm_ctx *c, const spamm_params *p, const void *dAh, con
 
 int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_t row1, double *out3) {
     if (!c || !dC || !out3) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->have_a || !c->have_b || c->a_pruned || c->b_pruned) return SPAMM_ESTATE;   // needs complete fp16 copies
     if (row0 < 0 || row1 > c->M || row0 >= row1 || row0 % 64 || row1 % 64 || c->N % 64 || c->K % 16)
         return SPAMM_EINVAL;
@@ -564,6 +602,7 @@ int spamm_error_vs_dense_f64(spamm_ctx *c, const float *dC, int64_t row0, int64_
 
 int spamm_dropped_bound(spamm_ctx *c, float tau, double *out) {
     if (!c || !out || tau != tau) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     Shape s;
     if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     int rc = set_device(c);
@@ -572,48 +611,26 @@ int spamm_dropped_bound(spamm_ctx *c, float tau, double *out) {
     if ((rc = ensure(c, c->tauws, tau_workspace_bytes()))) return rc;
     double *d = (double *)c->tauws.p;
     HIPCHK(c, launch_dropped_bound((const float *)c->nA.p, (const float *)c->nBt.p, s.nbM, s.nbK, s.nbN, tau, d,
-                                   c->stream));
+                                   nullptr, c->stream));
     double sq;
     if ((rc = copy_out(c, d, &sq, sizeof(sq)))) return rc;
     *out = sqrt(sq);
     return SPAMM_OK;
 }
 
-int spamm_mfma_ceiling(spamm_ctx *c, int random_operands, int iters, double *tflops, double *clock_ghz) {
-    if (!c || !tflops || !clock_ghz || iters <= 0 || iters > (1 << 20)) return SPAMM_EINVAL;
+int spamm_dropped_bound_tiles(spamm_ctx *c, float tau, double *host_out) {
+    if (!c || !host_out || tau != tau) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
+    if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     int rc = set_device(c);
     if (rc) return rc;
-    int n_wg = 0;
-    HIPCHK(c, hipDeviceGetAttribute(&n_wg, hipDeviceAttributeMultiprocessorCount, c->device));
-    if (n_wg <= 0 || n_wg > 4096) return SPAMM_EHIP;
-    // operands: 2048 vectors of 8 halves, zeros or uniform in [-1, 1) (a fixed LCG sequence)
-    std::vector<_Float16> h(2048 * 8);
-    uint32_t x = 12345u;
-    for (size_t i = 0; i < h.size(); i++) {
-        x = x * 1664525u + 1013904223u;
-        h[i] = random_operands ? (_Float16)(((float)(x >> 8) / 8388608.0f) - 1.0f) : (_Float16)0.0f;
-    }
-    const size_t in_bytes = h.size() * 2, out_bytes = (size_t)n_wg * 256 * 4, tr_bytes = (size_t)n_wg * 16;
-    if ((rc = ensure(c, c->staging, in_bytes + out_bytes + tr_bytes))) return rc;
-    char *base = (char *)c->staging.p;
-    HIPCHK(c, hipMemcpyAsync(base, h.data(), in_bytes, hipMemcpyHostToDevice, c->stream));
-    HIPCHK(c, hipStreamSynchronize(c->stream));
-    double best_ns = 0.0, best_clk = 0.0;
-    std::vector<unsigned long long> tr((size_t)n_wg * 2);
-    for (int rep = 0; rep < 3; rep++) {   // the clock settles over the first launches; keep the last
-        HIPCHK(c, launch_mfma_ceiling(base, (float *)(base + in_bytes), (unsigned long long *)(base + in_bytes + out_bytes),
-                                      n_wg, iters, c->stream));
-        if ((rc = copy_out(c, base + in_bytes + out_bytes, tr.data(), tr_bytes))) return rc;
-        double w = 0.0, k = 0.0;
-        for (int i = 0; i < n_wg; i++) { w += (double)tr[2 * i]; k += (double)tr[2 * i + 1]; }
-        best_ns = w / n_wg * 10.0;        // wall ticks are 10 ns
-        best_clk = k / n_wg;
-    }
-    if (best_ns <= 0.0) return SPAMM_EHIP;
-    const double flops = (double)iters * 16.0 * 32768.0 * 4.0 * n_wg;   // per MFMA 2*32*32*16, 4 waves per workgroup
-    *tflops = flops / best_ns * 1e-3;
-    *clock_ghz = best_clk / best_ns;
-    return SPAMM_OK;
+    const Shape s = shape_of(c);
+    const size_t nt = (size_t)s.nbM * s.nbN;
+    if ((rc = ensure(c, c->tauws, tau_workspace_bytes()))) return rc;
+    if ((rc = ensure(c, c->staging, nt * 8))) return rc;
+    HIPCHK(c, launch_dropped_bound((const float *)c->nA.p, (const float *)c->nBt.p, s.nbM, s.nbK, s.nbN, tau,
+                                   (double *)c->tauws.p, (double *)c->staging.p, c->stream));
+    return copy_out(c, c->staging.p, host_out, nt * 8);
 }
 
 // ---- input adapters (host side; getMatrixFromCSV / getMatrixFromMTX, tool.cu:282-366)
@@ -688,6 +705,7 @@ int spamm_load_mtx_f32(const char *path, int64_t rows, int64_t cols, int64_t ld,
 }
 
 static int tau_prepare(spamm_ctx *c, Shape *s) {
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->tile || !c->M || !c->K || !c->N || !c->nm_a || !c->nm_b) return SPAMM_ESTATE;   // both norm maps, same K and tile
     int rc = set_device(c);
     if (rc) return rc;
@@ -773,6 +791,7 @@ int spamm_tune_bisect(spamm_ctx *c, double expected, double tol, int max_rounds,
 
 int spamm_get_stats(spamm_ctx *c, spamm_stats *out) {
     if (!c || !out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     memset(out, 0, sizeof(*out));
     if (!c->have_gate) return SPAMM_ESTATE;
     int rc = set_device(c);
@@ -795,6 +814,7 @@ int spamm_get_stats(spamm_ctx *c, spamm_stats *out) {
 
 int spamm_get_normmap(spamm_ctx *c, int role, float *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->tile) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
     if (role == SPAMM_ROLE_A) {
@@ -810,6 +830,7 @@ int spamm_get_normmap(spamm_ctx *c, int role, float *host_out) {
 
 int spamm_get_counts(spamm_ctx *c, int32_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->have_gate) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
     return copy_out(c, c->counts.p, host_out, (size_t)s.nbM * s.nbN * 4);
@@ -817,6 +838,7 @@ int spamm_get_counts(spamm_ctx *c, int32_t *host_out) {
 
 int spamm_get_klist(spamm_ctx *c, uint16_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->have_gate) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
     // built from the bitmaps on demand: the multiply itself never reads per-tile lists
@@ -830,6 +852,7 @@ int spamm_get_klist(spamm_ctx *c, uint16_t *host_out) {
 
 int spamm_get_mask(spamm_ctx *c, uint64_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     if (!c->have_gate) return SPAMM_ESTATE;
     const Shape s = shape_of(c);
     return copy_out(c, c->mask.p, host_out, (size_t)s.nbM * s.nbN * s.words * 8);
@@ -837,6 +860,7 @@ int spamm_get_mask(spamm_ctx *c, uint64_t *host_out) {
 
 int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
     int rc = set_device(c);
     if (rc) return rc;
     int64_t rows, cols;

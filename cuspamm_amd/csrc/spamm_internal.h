@@ -89,11 +89,9 @@ hipError_t launch_normmap_ab(const void *X, bool in16, int64_t n, int tile, void
 hipError_t launch_error_vs_dense(const void *packedA, const void *packedB, int64_t M, int64_t K, int64_t N,
                                  int tile, const float *C, int64_t row0, int64_t row1, double *out3,
                                  hipStream_t s);
+// out1 += sum over tiles of s_ij^2, s_ij = sum_{k dropped} nA[i,k]*nB[k,j]; per_tile (optional): s_ij
 hipError_t launch_dropped_bound(const float *nA, const float *nBt, int64_t nbM, int64_t nbK, int64_t nbN,
-                                float tau, double *out1, hipStream_t s);
-// matrix-pipeline ceiling probe: n_wg workgroups issue iters x 16 MFMAs per wave on the 32 KiB of operands at `in`
-hipError_t launch_mfma_ceiling(const void *in, float *out, unsigned long long *trace, int n_wg, int iters,
-                               hipStream_t s);
+                                float tau, double *out1, double *per_tile, hipStream_t s);
 hipError_t launch_unpack(const void *packed, int64_t rows, int64_t cols, int tile, int role,
                          uint16_t *out, hipStream_t s);
 hipError_t launch_transpose_normmap(const float *nB, int64_t nbK, int64_t nbN, float *nBt,
@@ -149,6 +147,6 @@ hipError_t launch_tau_count(const float *nA, const float *nBt, int64_t nbM, int6
 
 hipError_t gemm_init();   // one-time kernel attribute set-up
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, hipStream_t s);
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, hipStream_t s);
 
 }  // namespace spamm

@@ -92,6 +92,20 @@ typedef struct spamm_ctx spamm_ctx;
 SPAMM_API int spamm_create(spamm_ctx **out, int device);
 SPAMM_API int spamm_destroy(spamm_ctx *ctx);
 
+/* Tuning options.  The defaults suit a whole MI355X; nothing here changes C, mask or counts.
+ *   SPAMM_OPT_NUM_XCD: number of XCDs (32 CUs sharing an L2) the GEMM schedule deals workgroups to:
+ *     1, 2, 4 or 8; 0 = derive from the device's CU count (what spamm_create does; a partitioned
+ *     device shows fewer).  Invalidates the gate of the last call.
+ *   SPAMM_OPT_GATE_CHUNK_WORDS: the gate walks K in chunks of at most this many 64-k-tile bitmap
+ *     words; 0 = as many as fit LDS (one chunk unless K / tile exceeds ~19 500 at tile 32).
+ *   SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's operand ring, 3..5; 0 = default (4).
+ * SPAMM_EINVAL for an unknown option or a value outside its range.  The reference has no such
+ * knobs: its launch shapes are compile-time constants (main.h:32-73). */
+#define SPAMM_OPT_NUM_XCD 1
+#define SPAMM_OPT_GATE_CHUNK_WORDS 2
+#define SPAMM_OPT_GEMM_RING 3
+SPAMM_API int spamm_set_option(spamm_ctx *ctx, int option, int value);
+
 /* Run all stages on a caller-provided hipStream_t (default: the context's own
  * stream).  Pass NULL to return to the context's stream. */
 SPAMM_API int spamm_set_stream(spamm_ctx *ctx, void *hip_stream);
@@ -122,8 +136,10 @@ SPAMM_API int spamm_multiply_f16(spamm_ctx *ctx, const spamm_params *p, const vo
  * SPAMM_FLAG_REUSE_A/B are rejected (SPAMM_EINVAL).  All contexts on one GPU share the array and it
  * keeps the last call's contents: calls that overlap in time on one GPU (two contexts, two
  * streams) race; issue them one after the other.  Afterwards the context's read-backs and stage
- * calls refer to this call's results; the next ordinary multiply / norm-map call returns to the
- * context's own workspace, whose contents (and REUSE state) are as it left them. */
+ * calls refer to this call's results -- until ANY context makes the next spamm_multiply_noalloc
+ * on the same GPU: from then on they return SPAMM_ESTATE for this context (the array now holds the
+ * other call's bytes).  The next ordinary multiply / norm-map call returns to the context's own
+ * workspace, whose contents (and REUSE state) are as it left them. */
 #define SPAMM_NOALLOC_WORKSPACE_BYTES (40u << 20)
 SPAMM_API int spamm_multiply_noalloc(spamm_ctx *ctx, const spamm_params *p, const float *dA, const float *dB,
                                      float *dC);
@@ -206,18 +222,13 @@ SPAMM_API int spamm_fill_decay_f32(spamm_ctx *ctx, float *dX, int64_t rows, int6
  * (multiples of 64; N a multiple of 64).  The dense product is never stored. */
 SPAMM_API int spamm_error_vs_dense_f64(spamm_ctx *ctx, const float *dC, int64_t row0, int64_t row1,
                                        double *out3);
-/* tau-derived bound on that error: sqrt(sum_ij (sum_{k dropped} nA[i,k]*nB[k,j])^2). */
+/* tau-derived bound on that error: sqrt(sum_ij s_ij^2) with s_ij = sum_{k dropped} nA[i,k]*nB[k,j],
+ * the bound on ||C_ij - (A B)_ij||_F of output tile (i,j).  spamm_dropped_bound_tiles returns the
+ * per-tile s_ij themselves, row-major [M/b x N/b] doubles in a HOST buffer (where the error sits,
+ * which the reference's single printed norm, tool.cu:6-24, does not tell).  Both use the norm maps
+ * of stage 1 and take tau as an argument (the gate need not have run). */
 SPAMM_API int spamm_dropped_bound(spamm_ctx *ctx, float tau, double *out);
-
-/* Measurement aid with no counterpart in the reference: the rate the matrix
- * pipeline sustains when every CU issues nothing but independent fp16
- * 32x32x16 MFMAs (iters x 16 per wave, one wave per SIMD), with all-zero
- * operands (random_operands = 0) or uniform [-1,1) operands (1).  The
- * sustained clock under MFMA load depends on the operand values, so the
- * second figure is the ceiling a GEMM on real data can approach; it is
- * reported next to the datasheet peak.  Synchronises. */
-SPAMM_API int spamm_mfma_ceiling(spamm_ctx *ctx, int random_operands, int iters, double *tflops,
-                                 double *clock_ghz);
+SPAMM_API int spamm_dropped_bound_tiles(spamm_ctx *ctx, float tau, double *host_out);
 
 /* Input adapters (host): dense CSV, one matrix row per line (getMatrixFromCSV,
  * tool.cu:329-366), and "row col val" triples, 1-based, first line skipped

@@ -58,6 +58,8 @@ def lib():
     L.orc_frob_diff_f32.argtypes = [_f32p, _f32p, _i64, _f64p]
     L.orc_dropped_bound.argtypes = [_f32p, _f32p, _i64, _i64, _i64, ctypes.c_float, _i64, _i64]
     L.orc_dropped_bound.restype = ctypes.c_double
+    L.orc_dropped_bound_tiles.argtypes = [_f32p, _f32p, _i64, _i64, _i64, ctypes.c_float, _f64p]
+    L.orc_dropped_bound_tiles.restype = None
     L.orc_tau_for_ratio.argtypes = [_f32p, _f32p, _i64, _i64, _i64, ctypes.c_double,
                                     ctypes.POINTER(ctypes.c_double)]
     L.orc_tau_for_ratio.restype = ctypes.c_float
@@ -217,6 +219,16 @@ def dropped_bound(nA, nB, tau, ti0=0, ti1=None):
         ti1 = nbM
     return float(lib().orc_dropped_bound(nA.reshape(-1), nB.reshape(-1), nbM, nbK, nbN,
                                          np.float32(tau), ti0, ti1))
+
+
+def dropped_bound_tiles(nA, nB, tau):
+    nA = np.ascontiguousarray(nA, dtype=np.float32)
+    nB = np.ascontiguousarray(nB, dtype=np.float32)
+    nbM, nbK = nA.shape
+    _, nbN = nB.shape
+    out = np.zeros(nbM * nbN, dtype=np.float64)
+    lib().orc_dropped_bound_tiles(nA.reshape(-1), nB.reshape(-1), nbM, nbK, nbN, np.float32(tau), out)
+    return out.reshape(nbM, nbN)
 
 
 def tau_for_ratio(nA, nB, ratio):

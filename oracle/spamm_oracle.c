@@ -397,6 +397,23 @@ ORC_API double orc_dropped_bound(const float *nA, const float *nB, int64_t nbM, 
     return sqrt(tot);
 }
 
+/* The same sums per output tile: out[i*nbN + j] = sum over dropped k of nA[i,k]*nB[k,j] (the bound
+ * on the Frobenius error of tile (i,j)); orc_dropped_bound is the root of the sum of their squares. */
+ORC_API void orc_dropped_bound_tiles(const float *nA, const float *nB, int64_t nbM, int64_t nbK,
+                                     int64_t nbN, float tau, double *out) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < nbM; i++) {
+        for (int64_t j = 0; j < nbN; j++) {
+            double s = 0;
+            for (int64_t k = 0; k < nbK; k++) {
+                volatile float p = nA[i * nbK + k] * nB[k * nbN + j];
+                if (!(p >= tau)) s += (double)nA[i * nbK + k] * (double)nB[k * nbN + j];
+            }
+            out[i * nbN + j] = s;
+        }
+    }
+}
+
 /* ---------------------------------------------------------- tau selection */
 
 static int cmp_float_desc(const void *a, const void *b) {

@@ -31,6 +31,73 @@ def test_library_exports_every_declared_symbol():
     assert L.spamm_version() >= 100
 
 
+def test_dev_library_is_separate_from_the_engine():
+    # measurement aids live in a library of their own: the engine exports no probe, and the aid's
+    # header declares exactly what its library exports
+    import cuspamm_amd as sp
+    from cuspamm_amd import dev
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "spamm_dev.h")).read(), flags=re.S)
+    syms = sorted(set(re.findall(r"\b(spamm_dev_[a-z0-9_]+)\s*\(", text)))
+    assert syms == ["spamm_dev_mfma_ceiling"]
+    D = dev.load_dev_library()
+    for name in syms:
+        assert hasattr(D, name), name
+    L = sp.load_library()
+    assert not hasattr(L, "spamm_mfma_ceiling") and not hasattr(L, "spamm_dev_mfma_ceiling")
+    assert D.spamm_dev_mfma_ceiling(0, 0, 0, None, None) == -1        # bad arguments: refused before any device call
+
+
+def test_option_values_match_header():
+    from cuspamm_amd import api
+    text = open(os.path.join(ROOT, "include", "spamm.h")).read()
+    opts = dict(re.findall(r"#define\s+SPAMM_(OPT_[A-Z_]+)\s+(\d+)", text))
+    assert set(opts) == {"OPT_NUM_XCD", "OPT_GATE_CHUNK_WORDS", "OPT_GEMM_RING"}
+    for name, value in opts.items():
+        assert getattr(api, name) == int(value), name
+    L = api.load_library()
+    assert L.spamm_set_option(None, 1, 8) == -1
+
+
+def test_engine_reads_no_environment_variables():
+    # tuning goes through spamm_set_option on a context, never through process-wide state
+    csrc = os.path.join(ROOT, "cuspamm_amd", "csrc")
+    for f in os.listdir(csrc):
+        if f.endswith((".hip", ".h")):
+            assert "getenv" not in open(os.path.join(csrc, f)).read(), f
+
+
+class _RecordingLib:
+    """Stands in for the loaded library: any entry point called is recorded (and none should be)."""
+    def __init__(self):
+        self.calls = []
+
+    def __getattr__(self, name):
+        def f(*a):
+            self.calls.append(name)
+            return 0
+        return f
+
+
+def test_wrapper_refuses_a_short_c_before_any_launch():
+    # the GEMM writes M x N floats through C's pointer: a smaller C must never reach the library
+    import torch
+    from cuspamm_amd import api
+    ctx = object.__new__(api.SpammContext)
+    ctx._lib, ctx._h, ctx._shape = _RecordingLib(), ctypes.c_void_p(1), None
+    A, B = torch.zeros((128, 64)), torch.zeros((64, 256))
+    for bad_c in (torch.zeros((128, 128)), torch.zeros((64, 256)), torch.zeros(128 * 256), torch.zeros((1, 128, 256))):
+        with pytest.raises(ValueError):
+            ctx.multiply(A, B, 64, 0.0, C=bad_c)
+        with pytest.raises(ValueError):
+            ctx.multiply_noalloc(A, B, 64, 0.0, bad_c)
+    with pytest.raises(ValueError):
+        ctx.multiply_noalloc(torch.zeros(128), B, 64, 0.0, torch.zeros((128, 256)))
+    with pytest.raises(ValueError):
+        ctx.multiply(A, torch.zeros((32, 256)), 64, 0.0)
+    assert ctx._lib.calls == []
+    ctx._h = ctypes.c_void_p()            # nothing to destroy
+
+
 def test_struct_layout_matches_header():
     import cuspamm_amd as sp
     assert ctypes.sizeof(sp.SpammParams) == 40

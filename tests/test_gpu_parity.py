@@ -92,6 +92,42 @@ def test_baseline_config1_a_equals_b(orc, ctx):
     assert 0.005 < ref["kept"] / 32 ** 3 < 0.03
 
 
+def test_reference_default_experiment(orc, ctx):
+    """The reference as checked out (para.h:1-14, cuSpAMM.cu:428-431): 2048^3, tile 32 (main.h:32),
+    both operands getDecayMatrixAlg(0.1, 0.1) (tool.cu:426-436), Norm = 1.548969, fp16 inputs
+    (USINGHALF 1) resident before the multiply."""
+    import torch
+    n, b, tau = 2048, 32, 1.548969
+    tab = orc.decay_table("ref_alg", n, c=0.1, v=0.1)
+    A = orc.fill_decay(n, n, tab, 0, random=False)
+    dA32 = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    ctx.fill_decay(dA32, tab, 0, random=False)                     # the device generator gives the same matrix
+    assert np.array_equal(dA32.cpu().numpy(), A)
+    hA = dA32.half()
+    hB = hA.clone()
+    C = torch.full((n, n), float("nan"), dtype=torch.float32, device="cuda")
+    ctx.multiply(hA, hB, b, tau, C=C)
+    ref = orc.spamm(A, A.copy(), b, tau)
+    assert np.array_equal(ctx.get_fp16(0), ref["hA"]) and np.array_equal(ctx.get_fp16(1), ref["hB"])
+    assert np.array_equal(ctx.get_normmap(0).view(np.uint32), ref["nA"].view(np.uint32))
+    assert np.array_equal(ctx.get_normmap(1).view(np.uint32), ref["nB"].view(np.uint32))
+    assert np.array_equal(ctx.get_mask(), ref["mask"])
+    assert np.array_equal(ctx.get_counts(), ref["counts"])
+    st = ctx.get_stats()
+    assert st.kept_products == ref["kept"] and 0.04 < st.kept_products / st.total_products < 0.06
+    Cg = C.cpu().numpy()
+    assert not np.isnan(Cg).any()
+    err, nrm, _ = orc.frob_diff(Cg, ref["C"])
+    assert err <= C_REL_TOL * nrm
+    # the tuner the reference runs on this matrix (tuneValidRate, tool.cu:438-490; main.h:35-38)
+    assert ctx.tune_bisect(0.75, 0.01, 20) == pytest.approx(orc.tune_bisect(ref["nA"], ref["nB"], 0.75, 0.01, 20))
+    # the pruned call and the A = B single pass give the same C bit for bit
+    C2 = ctx.multiply(hA, hB, b, tau, prune=True)
+    assert torch.equal(C2, C)
+    C3 = ctx.multiply(hA, hA, b, tau, a_eq_b=True)
+    assert torch.equal(C3, C)
+
+
 @pytest.mark.parametrize("name", ["exp_b32", "exp_b64_rect", "alg_b32", "exp_b128"])
 def test_against_committed_golden_vectors(ctx, name):
     import torch

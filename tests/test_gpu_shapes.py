@@ -80,15 +80,14 @@ def test_more_than_512_super_tiles_of_c(orc, ctx, M, n_sup_n, percents):
 
 
 @pytest.mark.parametrize("chunk_words", [1, 3])
-def test_gate_in_small_k_chunks_gives_the_same_lists(orc, ctx, monkeypatch, chunk_words):
+def test_gate_in_small_k_chunks_gives_the_same_lists(orc, ctx, chunk_words):
     """A macro tile's bitmaps normally fit a CU's LDS whole; beyond ~19 500 k tiles (tile 32) the
     gate walks k in chunks, twice.  Forcing chunks of 1 and 3 words (64 and 192 k tiles) sends
     ordinary shapes down that path: mask, counts, kept total and C must not change by a bit."""
     import torch
     import cuspamm_amd as sp
-    monkeypatch.setenv("SPAMM_GATE_CHUNK_WORDS", str(chunk_words))     # read once, when the context is created
     other = sp.SpammContext(0)
-    monkeypatch.delenv("SPAMM_GATE_CHUNK_WORDS")
+    other.set_option(sp.OPT_GATE_CHUNK_WORDS, chunk_words)
     try:
         for (M, K, N), tile, lam, ratio in [((512, 8192, 768), 32, 0.004, 0.3), ((1024, 12800, 512), 64, 0.001, 0.5),
                                             ((256, 33280, 384), 128, 0.0005, 0.4), ((320, 6432, 288), 32, 0.0, 1.0)]:
@@ -154,15 +153,14 @@ def test_non_finite_inputs_follow_ieee_compare(orc, ctx):
 
 
 @pytest.mark.parametrize("n_xcd", [1, 2, 4])
-def test_schedule_for_other_xcd_counts_gives_the_same_product(orc, ctx, n_xcd, monkeypatch):
+def test_schedule_for_other_xcd_counts_gives_the_same_product(orc, ctx, n_xcd):
     """The GEMM schedule is built for the device's XCD count (8 on a whole MI355X); a partitioned
     device, or one that is not whole XCDs of 32 CUs, gets 4 / 2 / 1 sequences.  The schedule only
     decides where and when a macro tile runs: mask and C must not change by a bit."""
     import torch
     import cuspamm_amd as sp
-    monkeypatch.setenv("SPAMM_NUM_XCD", str(n_xcd))          # read once, when the context is created
     other = sp.SpammContext(0)
-    monkeypatch.delenv("SPAMM_NUM_XCD")
+    other.set_option(sp.OPT_NUM_XCD, n_xcd)
     try:
         # (the last case is a narrow band over 128 super tiles: the grouped row-major deal)
         for (M, K, N), tile, lam, ratio in [((2304, 1024, 4352), 64, 0.004, 0.3), ((1280, 512, 768), 32, 0.01, 0.5),

@@ -100,6 +100,16 @@ def test_error_report_matches_checker(orc, ctx):
         gb = ctx.dropped_bound(tau)
         assert abs(gb - bound) <= 1e-9 * max(bound, 1e-30)
         assert ge <= gb * (1 + 1e-4) + 1e-5 * gd
+        # per output tile: the dropped sums themselves, against the checker's, and consistent with
+        # the scalar (root of the sum of squares, whole matrix and a row range)
+        gt = ctx.dropped_bound_tiles(tau)
+        ot = orc.dropped_bound_tiles(ctx.get_normmap(0), ctx.get_normmap(1), tau)
+        assert gt.shape == ot.shape == (n // tile, n // tile)
+        assert np.all(np.abs(gt - ot) <= 1e-12 * np.maximum(ot, 1e-300)), np.abs(gt - ot).max()
+        assert np.array_equal(gt == 0, ot == 0)
+        assert abs(np.sqrt((gt ** 2).sum()) - gb) <= 1e-9 * max(gb, 1e-30)
+        part = orc.dropped_bound(ctx.get_normmap(0), ctx.get_normmap(1), tau, 2, 5)
+        assert abs(np.sqrt((gt[2:5] ** 2).sum()) - part) <= 1e-9 * max(part, 1e-30)
         # row range
         ge2, gd2, _ = ctx.error_vs_dense(C, 128, 256)
         e2, d2, _ = orc.frob_diff(C.cpu().numpy()[128:256], dense[128:256])

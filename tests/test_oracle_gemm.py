@@ -123,6 +123,23 @@ def test_dropped_bound_hand_worked(orc):
     assert orc.dropped_bound(np.array([[3.0]], dtype=np.float32), np.array([[third]], dtype=np.float32), 1.0) == 0.0
 
 
+def test_dropped_bound_tiles_hand_worked(orc):
+    # same map as above: per-tile dropped sums at tau = 10 are 7, 10 / 4, 8; at tau = 8: 7, 2 / 4, 0
+    nA = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)
+    nB = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    assert np.array_equal(orc.dropped_bound_tiles(nA, nB, 10.0), np.array([[7.0, 10.0], [4.0, 8.0]]))
+    assert np.array_equal(orc.dropped_bound_tiles(nA, nB, 8.0), np.array([[7.0, 2.0], [4.0, 0.0]]))
+    assert np.array_equal(orc.dropped_bound_tiles(nA, nB, 0.0), np.zeros((2, 2)))
+    # everything dropped: the tile sums are the plain product of the norm maps
+    assert np.array_equal(orc.dropped_bound_tiles(nA, nB, 1e9), nA.astype(np.float64) @ nB.astype(np.float64))
+    # and the scalar bound is the root of the sum of their squares, row range by row range
+    rng = np.random.default_rng(5)
+    a, b = rng.random((5, 7), dtype=np.float32), rng.random((7, 4), dtype=np.float32)
+    t = orc.dropped_bound_tiles(a, b, 0.3)
+    assert orc.dropped_bound(a, b, 0.3) == pytest.approx(np.sqrt((t ** 2).sum()), rel=1e-14)
+    assert orc.dropped_bound(a, b, 0.3, 2, 4) == pytest.approx(np.sqrt((t[2:4] ** 2).sum()), rel=1e-14)
+
+
 def test_row_slab_interface(orc):
     b, n = 32, 128
     A, B = _inputs(orc, n, n, n, 0.02)

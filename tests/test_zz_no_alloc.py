@@ -69,6 +69,43 @@ def test_noalloc_leaves_the_contexts_own_workspace_alone(orc, ctx):
     assert np.array_equal(ctx.get_mask(), orc.spamm(A1, B, 64, 0.5)["mask"])
 
 
+def test_noalloc_results_go_stale_when_another_context_uses_the_array(orc, ctx):
+    """All contexts on a GPU share the one fixed array: after another context's noalloc call this
+    context's read-backs and stage calls must refuse (SPAMM_ESTATE) instead of handing out the other
+    call's bytes; an ordinary multiply brings the context back to its own workspace."""
+    import torch
+    import cuspamm_amd as sp
+    A, B = _case(orc, 256, 256, 256, 0.02, (1, 2))
+    A2, B2 = _case(orc, 384, 128, 256, 0.02, (3, 4))
+    dA, dB = _dev(A), _dev(B)
+    got = torch.empty((256, 256), dtype=torch.float32, device="cuda")
+    other = sp.SpammContext(0)
+    try:
+        ctx.multiply_noalloc(dA, dB, 64, 0.1, got)
+        ref = orc.spamm(A, B, 64, 0.1)
+        _check_against(ctx, orc, got, ref, "first context")
+        got2 = torch.empty((384, 256), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        other.multiply_noalloc(_dev(A2), _dev(B2), 64, 0.1, got2)
+        _check_against(other, orc, got2, orc.spamm(A2, B2, 64, 0.1), "second context")
+        for call in (ctx.get_mask, ctx.get_counts, ctx.get_stats, lambda: ctx.get_normmap(0), lambda: ctx.gate(0.1),
+                     lambda: ctx.gemm_gated(got), lambda: ctx.dropped_bound(0.1), lambda: ctx.tau_for_ratio(0.5)):
+            with pytest.raises(sp.SpammError) as ei:
+                call()
+            assert ei.value.code == sp.api.ESTATE
+        # the other context's results are still its own
+        assert np.array_equal(other.get_mask(), orc.spamm(A2, B2, 64, 0.1)["mask"])
+        # an ordinary call returns to the own workspace; a new noalloc call makes the results current again
+        C = ctx.multiply(dA, dB, 64, 0.1)
+        assert torch.equal(C, got) and np.array_equal(ctx.get_mask(), ref["mask"])
+        ctx.multiply_noalloc(dA, dB, 64, 0.1, got)
+        assert np.array_equal(ctx.get_mask(), ref["mask"])
+        with pytest.raises(sp.SpammError):
+            other.get_mask()
+    finally:
+        other.close()
+
+
 def test_noalloc_a_equals_b(orc, ctx):
     import torch
     n = 512
