@@ -19,6 +19,7 @@ namespace spamm {
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4n __attribute__((ext_vector_type(4)));
+typedef _Float16 half8n __attribute__((ext_vector_type(8)));
 
 // Convert two floats to fp16 (round-to-nearest-even), add their squares to s
 // in order (a then b) and return the packed pair.
@@ -61,7 +62,7 @@ __device__ __forceinline__ float butterfly64(float v) {
 // (The phased A role is held to three waves per SIMD: it gains more from a third resident
 // workgroup than it loses to a few spilled registers; the B role would spill far more.)
 template <int B, int ROLE, int SW, bool IN16, int PH = 1>
-__global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
+__global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT, uint4 *__restrict__ packed2,
@@ -70,13 +71,19 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
     constexpr int TPS = SW / B;           // tiles per strip
     constexpr int TPP = TPS / PH;         // tiles per phase (resident in LDS together)
     static_assert(TPP * PH == TPS && TPP >= 1, "phases must divide the strip's tiles");
-    // Lane -> element mapping.  PH = 1: a wave-wide load covers whole strip rows (LPR lanes
-    // each).  PH > 1: the waves are split between the phases' tiles (WPP waves per phase), a
+    // Lane -> element mapping.
+    // fp32 input, PH = 1: a wave-wide load covers whole strip rows (LPR lanes each, 4 columns a
+    // lane).  PH > 1: the waves are split between the phases' tiles (WPP waves per phase), a
     // wave-wide load covers rows of its own tiles only (the waves of the other phases read the
     // neighbouring segments of the same rows at the same time), and a phase is staged by whole
     // waves.
-    constexpr int WPP = 4 / PH;                        // waves per phase
-    constexpr int LPR = (PH > 1 ? TPP * B : SW) / 4;   // lanes across one row of the wave's columns
+    // fp16 input (IN16): a lane takes 8 columns (16 bytes), the strip is 512 columns wide and every
+    // wave-wide load is one whole strip row (1 KiB) whatever PH is; a lane's columns lie in one
+    // tile, and in phase ph only the lanes of that phase's tiles stage their data.
+    constexpr int EPL = IN16 ? 8 : 4;                  // columns per lane
+    static_assert(!IN16 || SW == 512, "fp16 input: 64 lanes x 8 columns");
+    constexpr int WPP = IN16 ? 4 : 4 / PH;             // waves that share a row range
+    constexpr int LPR = IN16 ? 64 : (PH > 1 ? TPP * B : SW) / 4;   // lanes across one row of the wave's columns
     constexpr int RH = 64 / LPR;                       // rows per wave-wide load
     constexpr int GSTEP = WPP * RH;                    // 8-row groups between a lane's groups
     static_assert(PH == 1 || PH == 2 || PH == 4, "phases are made of whole waves");
@@ -96,34 +103,35 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
     const int64_t I = blockIdx.x / nstrip;            // tile row of the strip
     const int64_t sc = blockIdx.x % nstrip;
     const int64_t col0 = sc * SW;
-    const int cl = (wave / WPP) * (TPP * B) + 4 * (lane % LPR);   // first column of this lane inside the strip
+    const int cl = IN16 ? EPL * lane : (wave / WPP) * (TPP * B) + 4 * (lane % LPR);   // first column of this lane inside the strip
     const int g0 = (wave % WPP) * RH + lane / LPR;    // first 8-row group of this lane; then every GSTEP-th
     const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
     const bool valid = col0 + cl < cols;
-    // IN16: the input already is fp16 (the reference's own input type, para.h:1); the
-    // conversion below is then the identity and only the packing and the norms remain
     const int64_t eoff = (I * B) * ld + col0 + cl;
 
-    f32x4 v[NGW][8];
+    // fp32 input: v holds the lane's elements; fp16 input (the reference's own input type,
+    // para.h:1): h16 holds them as loaded -- the conversion is then the identity and only the
+    // packing and the norms remain.
+    f32x4 v[IN16 ? 1 : NGW][8];
+    u32x4n h16[IN16 ? NGW : 1][8];
     if (IN16) {
         // every lane loads unconditionally (a lane beyond the last column reads the strip's first
-        // column instead and zeroes the values afterwards): with the loads inside a branch the
+        // columns instead and zeroes the values afterwards): with the loads inside a branch the
         // compiler waits for each one before it issues the next
-        typedef _Float16 half4v __attribute__((ext_vector_type(4)));
         const _Float16 *src = static_cast<const _Float16 *>(Xv) + (valid ? eoff : (I * B) * ld + col0);
-        half4v hv[NGW][8];
 #pragma unroll
         for (int i = 0; i < NGW; i++)
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                hv[i][j] = __builtin_nontemporal_load(
-                    reinterpret_cast<const half4v *>(src + (int64_t)(8 * (g0 + GSTEP * i) + j) * ld));
+            for (int j = 0; j < 8; j++) {
+                h16[i][j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4n *>(src + (int64_t)(8 * (g0 + GSTEP * i) + j) * ld));
+            }
+        if (!valid) {
 #pragma unroll
-        for (int i = 0; i < NGW; i++)
+            for (int i = 0; i < NGW; i++)
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                v[i][j] = valid ? f32x4{(float)hv[i][j].x, (float)hv[i][j].y, (float)hv[i][j].z, (float)hv[i][j].w}
-                                : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int j = 0; j < 8; j++) h16[i][j] = u32x4n{0u, 0u, 0u, 0u};
+        }
     } else {
 #pragma unroll
         for (int i = 0; i < NGW; i++)
@@ -137,6 +145,10 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
                         reinterpret_cast<const f32x4 *>(static_cast<const float *>(Xv) + eoff + (int64_t)r * ld));
             }
     }
+    // LDS position of the 16-byte vector of free index x inside a k-group segment.  The fp16-input
+    // B role writes 8 neighbouring x per lane, lanes 128 bytes apart: the low three bits of x are
+    // xor-ed with the next three so that the lanes of one store spread over the banks.
+    auto vpos = [](int x, bool swz) -> int { return swz ? (x ^ ((x >> 3) & 7)) : x; };
 
     // ROLE 2 = the same matrix is both operands (A = B): one read of X, both packed layouts and
     // both norm maps (A role first -> packed/nm, then B role -> packed2/nm2/nmT), LDS reused.
@@ -144,6 +156,21 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
         const int q = cin / 8, h = (cin % 8) / 4;
         if (PH > 1 && t / TPP != ph) return;
         const int t = (cl / B) % TPP;      // tile inside the phase
+        if constexpr (IN16) {
+            // the lane's 16 bytes are one whole chunk (8 consecutive k of row r): already a packed vector
+#pragma unroll
+            for (int i = 0; i < NGW; i++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int r = 8 * (g0 + GSTEP * i) + j;
+                    const half8n hv = __builtin_bit_cast(half8n, h16[i][j]);
+                    float s8 = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) { const float f = (float)hv[e]; s8 = s8 + f * f; }
+                    *reinterpret_cast<u32x4n *>(s_pack + t * TS + q * QS + r * 16) = h16[i][j];
+                    s_chunk[t * CH + r * PITCH + q] = s8;
+                }
+        } else {
 #pragma unroll
         for (int i = 0; i < NGW; i++)
 #pragma unroll
@@ -166,10 +193,36 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
                 *reinterpret_cast<uint2 *>(s_pack + t * TS + q * QS + r * 16 + h * 8) = o;
                 if (h) s_chunk[t * CH + r * PITCH + q] = s8;
             }
+        }
     };
     auto stage_b = [&](int ph) {
         if (PH > 1 && t / TPP != ph) return;
         const int t = (cl / B) % TPP;      // tile inside the phase
+        if constexpr (IN16) {
+            // the lane holds 8 rows (one k-group) x 8 columns: transposed in registers into 8
+            // k-contiguous vectors, one per column
+#pragma unroll
+            for (int i = 0; i < NGW; i++) {
+                const int kg = g0 + GSTEP * i;
+                half8n rows[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) rows[j] = __builtin_bit_cast(half8n, h16[i][j]);
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    half8n o;
+                    float sc_ = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        o[j] = rows[j][c];
+                        const float f = (float)rows[j][c];
+                        sc_ = sc_ + f * f;
+                    }
+                    *reinterpret_cast<u32x4n *>(s_pack + t * TS + kg * QS + vpos(cin + c, true) * 16) =
+                        __builtin_bit_cast(u32x4n, o);
+                    s_chunk[t * CH + (cin + c) * PITCH + kg] = sc_;
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < NGW; i++) {
             const int kg = g0 + GSTEP * i;
@@ -197,6 +250,7 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
                 s_chunk[t * CH + (cin + c) * PITCH + kg] = s[c];
             }
         }
+        }
     };
     // packed tiles out (256 threads x 16 bytes = 4 KiB per step, contiguous per tile)
     __shared__ int s_skip[TPP];
@@ -207,7 +261,7 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0) ? 3 : 1) void k_normmap(
             const int tt = vi / VPT, iv = vi % VPT;
             const int64_t Jt = sc * TPS + ph * TPP + tt;
             if (Jt < nbc && !(prune && s_skip[tt])) {
-                const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + (iv % B) * 16);
+                const uint4 d = *reinterpret_cast<const uint4 *>(s_pack + tt * TS + (iv / B) * QS + vpos(iv % B, IN16 && as_b) * 16);
                 const int64_t tile = as_b ? Jt * nbr + I : I * nbc + Jt;
                 __builtin_nontemporal_store(*reinterpret_cast<const u32x4n *>(&d), reinterpret_cast<u32x4n *>(pk + tile * VPT + iv));
             }
@@ -358,13 +412,14 @@ static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int 
                                  float *nmT, hipStream_t s, void *packed2 = nullptr, float *nm2 = nullptr,
                                  const float *rowmax = nullptr, float tau_skip = 0.0f) {
     const int64_t nbr = rows / tile, nbc = cols / tile;
-    const int sw = 256;
-    const int64_t nstrip = (cols + sw - 1) / sw;
+    constexpr int SW = IN16 ? 512 : 256;              // strip width: a wave-wide load is 1 KiB of one row
+    const int64_t nstrip = (cols + SW - 1) / SW;
     const unsigned grid = (unsigned)(nbr * nstrip);
+    // phases: tiles of a strip resident in LDS together take ~42 KiB at most (three workgroups per CU)
     switch (tile) {
-        case 32: k_normmap<32, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
-        case 64: k_normmap<64, ROLE, 256, IN16><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
-        case 128: k_normmap<128, ROLE, 256, IN16, 2><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 32: k_normmap<32, ROLE, SW, IN16, 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 64: k_normmap<64, ROLE, SW, IN16, IN16 ? 2 : 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 128: k_normmap<128, ROLE, SW, IN16, IN16 ? 4 : 2><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
