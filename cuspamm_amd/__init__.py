@@ -17,6 +17,7 @@ from .api import (  # noqa: F401
     OPT_NUM_XCD,
     OPT_GATE_CHUNK_WORDS,
     OPT_GEMM_RING,
+    OPT_GEMM_SHAPE,
     SpammContext,
     SpammError,
     SpammParams,

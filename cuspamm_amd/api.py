@@ -19,7 +19,7 @@ FLAG_REUSE_A = 4
 FLAG_REUSE_B = 8
 FLAG_PRUNE = 16
 
-OPT_NUM_XCD, OPT_GATE_CHUNK_WORDS, OPT_GEMM_RING = 1, 2, 3
+OPT_NUM_XCD, OPT_GATE_CHUNK_WORDS, OPT_GEMM_RING, OPT_GEMM_SHAPE = 1, 2, 3, 4
 
 OK, EINVAL, ENOMEM, EHIP, ESTATE, ENODEV, ELIMIT = 0, -1, -2, -3, -4, -5, -6
 NOALLOC_WORKSPACE_BYTES = 40 << 20

@@ -18,6 +18,7 @@
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "spamm_internal.h"
 
@@ -401,10 +402,335 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// The same multiply with a workgroup per HALF macro tile: 128 rows x 256 columns of C, 4 waves
+// (2 x 2), each wave 64 x 128 = 2 x 4 MFMA blocks = 128 accumulator registers, so two workgroups
+// (two waves per SIMD) share a CU: one workgroup's prologue, epilogue, barriers and LDS reads sit
+// under the other's MFMAs, and the work units are half as long (finer tail).  The price is the B
+// part of a stage staged once per half: 24 KiB per 2.1 Mflop instead of 32 KiB per 4.2 Mflop.
+// Lists, masks and the order of accumulation are the macro tile's, so C is bit-identical to
+// k_gemm's.  Workgroup pair (2 q, 2 q + 1) of an XCD's sequence takes the upper and lower half of
+// the XCD's q-th macro tile.
+constexpr int HALF_RING = 3;      // stages of the half shape's ring: 3 x 24 KiB, two workgroups per CU
+constexpr int W8_RING = 4;        // stages of the eight-wave shape's ring: 4 x 32 KiB, one workgroup per CU
+
+// NWR wave rows of 64 rows of C each: 2 = the half shape above, 4 = a whole macro tile by eight
+// waves (4 x 2; the same 32 KiB per stage as k_gemm, but two waves per SIMD).
+template <int B, int NWR>
+struct HalfCfg {
+    using G = GemmCfg<B>;
+    static constexpr int NW = 2 * NWR;                       // waves per workgroup
+    static constexpr int MR = 64 * NWR, WR = 64, NRB = 2;
+    static constexpr int MTA = MR / B > 0 ? MR / B : 1;      // A slots (tile rows) of a workgroup
+    static constexpr int PARTS = 256 / MR;                   // workgroups per macro tile
+    static constexpr int A_BYTES = MR * G::KS * 2;           // 8 or 16 KiB
+    static constexpr int B_BYTES = 256 * G::KS * 2;          // 16 KiB
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;    // 24 or 32 KiB
+    static constexpr int CHWA = A_BYTES / 1024 / NW;         // 1 KiB chunks per wave per stage: A part (2),
+    static constexpr int CHWB = B_BYTES / 1024 / NW;         // B part (4 or 2)
+    static constexpr int GSB = G::CPS < CHWB ? G::CPS : CHWB;   // B chunks per load group (share a tile)
+    static constexpr int NGB = CHWB / GSB;
+    static constexpr int LPW = CHWA + CHWB;                  // loads per wave per stage (6 or 4)
+    static constexpr int TRW = WR / B > 0 ? WR / B : 1;      // tile rows a wave touches
+    static constexpr int RBR = NRB / TRW;                    // MFMA row blocks per tile row of a wave
+    static_assert(G::CPS >= CHWA && CHWA == 2, "a wave's two A chunks lie in one slot");
+};
+
+template <int B, int NBUF, int NWR>
+__global__ __launch_bounds__(128 * NWR, NWR == 2 ? 2 : 1) void k_gemm_half(const unsigned char *__restrict__ pA,
+                                                      const unsigned char *__restrict__ pB,
+                                                      const MacroEntry *__restrict__ macro_list,
+                                                      const int32_t *__restrict__ macro_count,
+                                                      const int32_t *__restrict__ order,
+                                                      const int32_t *__restrict__ sched, int P, int n_xcd, int nbM,
+                                                      int nbK, int nbN, int nMacN, int64_t M, int64_t N,
+                                                      float *__restrict__ C) {
+    using G = GemmCfg<B>;
+    using H = HalfCfg<B, NWR>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    typedef const __attribute__((address_space(4))) u32x4 *entry_ptr;   // scalar (SMEM) loads
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int xcd = blockIdx.x % n_xcd, q2 = blockIdx.x / n_xcd;
+    const int q = q2 / H::PARTS, hf = q2 % H::PARTS;
+    const int ntot = __builtin_amdgcn_readfirstlane(sched[MAX_XCD + xcd]);
+    if (q >= ntot) return;
+    const int32_t *seq = order + (int64_t)xcd * P;
+    const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
+    const int mi = macro / nMacN, mj = macro % nMacN;
+    const int64_t row_half = (int64_t)mi * 256 + hf * H::MR;            // first row of C of this workgroup
+    if (row_half >= M) return;                                          // the lower half lies beyond the matrix
+    const int U = __builtin_amdgcn_readfirstlane(macro_count[2 * macro]);
+    const int Ufull = __builtin_amdgcn_readfirstlane(macro_count[2 * macro + 1]);
+    entry_ptr ents = (entry_ptr)(uintptr_t)(macro_list + (int64_t)macro * nbK);
+    const int S = U * G::NSPE, Sfull = Ufull * G::NSPE;
+    const uint32_t lds_base =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+    if (S == 0) {     // nothing kept in this macro tile: this half's zeros
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int64_t c0 = (int64_t)mj * 256 + lane * 4;
+        if (c0 < N)
+            for (int r = wave; r < H::MR && row_half + r < M; r += H::NW)
+                __builtin_nontemporal_store(zero, reinterpret_cast<f32x4 *>(C + (row_half + r) * N + c0));
+        return;
+    }
+
+    f32x16 acc[H::NRB][4];
+#pragma unroll
+    for (int r = 0; r < H::NRB; r++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[r][c][i] = 0.0f;
+
+    {
+        // ---- staging: a wave copies 2 consecutive 1 KiB chunks of the A part (one slot) and 4 of
+        // the B part (NGB groups of GSB chunks, each group inside one slot).  Clamping as in k_gemm.
+        const int chunkA0 = wave * H::CHWA;
+        const int slotA = chunkA0 / G::CPS, withinA = chunkA0 % G::CPS;
+        int tiA = mi * G::MT + hf * H::MTA + slotA;
+        tiA = tiA < nbM ? tiA : nbM - 1;
+        const unsigned char *rowA = pA + (int64_t)tiA * nbK * G::TILE_BYTES + withinA * 1024;
+        const uint32_t ldsA = lds_base + slotA * G::SLOT_BYTES + withinA * 1024;
+        const unsigned char *rowB[H::NGB];
+        uint32_t ldsB[H::NGB];
+        int slotB[H::NGB];
+#pragma unroll
+        for (int g = 0; g < H::NGB; g++) {
+            const int chunk0 = wave * H::CHWB + g * H::GSB;
+            const int slot = chunk0 / G::CPS, within0 = chunk0 % G::CPS;
+            int tj = mj * G::MT + slot;
+            tj = tj < nbN ? tj : nbN - 1;
+            rowB[g] = pB + (int64_t)tj * nbK * G::TILE_BYTES + within0 * 1024;
+            ldsB[g] = lds_base + H::A_BYTES + slot * G::SLOT_BYTES + within0 * 1024;
+            slotB[g] = slot;
+        }
+        const uint32_t voff = lane * 16;
+
+        auto stage_k = [&](int t) -> uint32_t {
+            const int tc = t < S ? t : S - 1;
+            return ents[tc / G::NSPE].x;
+        };
+        struct StageAddr {
+            int64_t koff;
+            uint32_t boff;
+        };
+        auto stage_addr = [&](int t, uint32_t k) -> StageAddr {
+            const int tc = t < S ? t : S - 1;
+            StageAddr sa;
+            sa.koff = (int64_t)k * G::TILE_BYTES + (tc % G::NSPE) * G::SLOT_BYTES;
+            sa.boff = (uint32_t)(t % NBUF) * H::STAGE_BYTES;
+            return sa;
+        };
+        // load i of a stage: 0, 1 = the wave's A chunks, 2..5 = its B chunks
+        auto issue_one = [&](const StageAddr &sa, auto idx) {
+            constexpr int i = decltype(idx)::value;
+            if constexpr (i < H::CHWA) {
+                dma_load<i * 1024>(rowA + sa.koff, voff, ldsA + sa.boff);
+            } else {
+                constexpr int g = (i - H::CHWA) / H::GSB, j = (i - H::CHWA) % H::GSB;
+                dma_load<j * 1024>(rowB[g] + sa.koff, voff, ldsB[g] + sa.boff);
+            }
+        };
+        // same, but a slot no kept product of this half needs is not fetched (cache-resident placeholder)
+        auto issue_needed = [&](const StageAddr &sa, uint32_t needA, uint32_t needB, auto idx) {
+            constexpr int i = decltype(idx)::value;
+            // (the choice is scalar arithmetic on purpose: the address must stay in scalar registers)
+            if constexpr (i < H::CHWA) {
+                const int64_t on = -(int64_t)((needA >> slotA) & 1u);
+                dma_load<i * 1024>(pA + (((rowA - pA) + sa.koff) & on), voff, ldsA + sa.boff);
+            } else {
+                constexpr int g = (i - H::CHWA) / H::GSB, j = (i - H::CHWA) % H::GSB;
+                const int64_t on = -(int64_t)((needB >> slotB[g]) & 1u);
+                dma_load<j * 1024>(pB + (((rowB[g] - pB) + sa.koff) & on), voff, ldsB[g] + sa.boff);
+            }
+        };
+#define SPAMM_ISSUE(sa, i) issue_one(sa, std::integral_constant<int, i>{})
+#define SPAMM_ISSUE_N(sa, na, nb_, i) issue_needed(sa, na, nb_, std::integral_constant<int, i>{})
+        // (loads 4 and 5 exist in the half shape only)
+#define SPAMM_ISSUE_X(sa, i) do { if constexpr (i < H::LPW) issue_one(sa, std::integral_constant<int, (i < H::LPW ? i : 0)>{}); } while (0)
+#define SPAMM_ISSUE_NX(sa, na, nb_, i) do { if constexpr (i < H::LPW) issue_needed(sa, na, nb_, std::integral_constant<int, (i < H::LPW ? i : 0)>{}); } while (0)
+        auto issue_all = [&](const StageAddr &sa) {
+            SPAMM_ISSUE(sa, 0); SPAMM_ISSUE(sa, 1); SPAMM_ISSUE(sa, 2);
+            SPAMM_ISSUE(sa, 3); SPAMM_ISSUE_X(sa, 4); SPAMM_ISSUE_X(sa, 5);
+        };
+        // the ring protocol and its vmcnt invariant are k_gemm's, with LPW = 6 loads per wave per stage
+        auto sync_next = [&]() {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(H::LPW * (NBUF - 2), 0));
+            __syncthreads();
+        };
+        auto frag_off = [&](int first, int blk, int kk) -> int {     // `first`: the wave's first row / column
+            const int off = first + blk * 32;
+            return (off / B) * G::SLOT_BYTES + (((2 * kk + (lane >> 5)) * B) + off % B + (lane & 31)) * 16;
+        };
+        auto load_frags = [&](half8 (&af)[H::NRB], half8 (&bf)[4], int t, int kk) {
+            const unsigned char *bufA = smem + (t % NBUF) * H::STAGE_BYTES;
+            const unsigned char *bufB = bufA + H::A_BYTES;
+#pragma unroll
+            for (int r = 0; r < H::NRB; r++) af[r] = *reinterpret_cast<const half8 *>(bufA + frag_off(wr * H::WR, r, kk));
+#pragma unroll
+            for (int c = 0; c < 4; c++) bf[c] = *reinterpret_cast<const half8 *>(bufB + frag_off(wc * 128, c, kk));
+        };
+
+        // ---- prologue: stages 0..NBUF-2 and the first two loads of stage NBUF-1
+#pragma unroll
+        for (int t = 0; t < NBUF - 1; t++) issue_all(stage_addr(t, stage_k(t)));
+        StageAddr sa_tail = stage_addr(NBUF - 1, stage_k(NBUF - 1));
+        SPAMM_ISSUE(sa_tail, 0); SPAMM_ISSUE(sa_tail, 1);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(H::LPW * (NBUF - 2) + 2, 0));
+        __syncthreads();
+        int t = 0;
+#define SPAMM_MFMA(A, Bv, r, c) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[r], Bv[c], acc[r][c], 0, 0, 0)
+#define SPAMM_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define SPAMM_LDA(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufA + frag_off(wr * H::WR, blk, kk))
+#define SPAMM_LDB(dst, blk, kk) dst = *reinterpret_cast<const half8 *>(bufB + frag_off(wc * 128, blk, kk))
+        half8 a0[H::NRB], b0[4], a1[H::NRB], b1[4];
+        load_frags(a0, b0, 0, 0);
+        // ---- loop 1: entries kept by all tiles of the macro tile, branch-free; 8 MFMAs per k step,
+        // the 6 LDS reads of the next k step and the stage's 6 global->LDS loads between them
+        if (Sfull > 0) {
+            uint32_t knext = stage_k(NBUF);
+            for (; t < Sfull; t++) {
+                const StageAddr sa_new = stage_addr(t + NBUF, knext);
+                SPAMM_FENCE();
+                {
+                    const unsigned char *bufA = smem + (t % NBUF) * H::STAGE_BYTES;
+                    const unsigned char *bufB = bufA + H::A_BYTES;
+                    SPAMM_MFMA(a0, b0, 0, 0); SPAMM_LDA(a1[0], 0, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 0, 1); SPAMM_LDB(b1[0], 0, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 2); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 0, 2); SPAMM_LDB(b1[1], 1, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 0, 3); SPAMM_LDB(b1[2], 2, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 3); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 1, 0); SPAMM_LDB(b1[3], 3, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 1, 1); SPAMM_LDA(a1[1], 1, 1); SPAMM_FENCE();
+                    SPAMM_ISSUE_X(sa_tail, 4); SPAMM_FENCE();
+                    SPAMM_MFMA(a0, b0, 1, 2); SPAMM_MFMA(a0, b0, 1, 3); SPAMM_FENCE();
+                    SPAMM_ISSUE_X(sa_tail, 5); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 0, 0); SPAMM_MFMA(a1, b1, 0, 1); SPAMM_MFMA(a1, b1, 0, 2); SPAMM_MFMA(a1, b1, 0, 3);
+                    SPAMM_FENCE();
+                }
+                sync_next();
+                SPAMM_FENCE();
+                knext = stage_k(t + 1 + NBUF);
+                sa_tail = sa_new;
+                SPAMM_FENCE();
+                {
+                    const unsigned char *bufA = smem + ((t + 1) % NBUF) * H::STAGE_BYTES;
+                    const unsigned char *bufB = bufA + H::A_BYTES;
+                    SPAMM_MFMA(a1, b1, 1, 0); SPAMM_LDA(a0[0], 0, 0); SPAMM_LDB(b0[0], 0, 0); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 1, 1); SPAMM_LDB(b0[1], 1, 0); SPAMM_LDB(b0[2], 2, 0); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 1, 2); SPAMM_LDB(b0[3], 3, 0); SPAMM_FENCE();
+                    SPAMM_ISSUE(sa_tail, 1); SPAMM_FENCE();
+                    SPAMM_MFMA(a1, b1, 1, 3); SPAMM_LDA(a0[1], 1, 0); SPAMM_FENCE();
+                }
+            }
+        }
+        // ---- loop 2: entries kept by some tiles only; this half multiplies exactly the pairs of its
+        // tile rows whose bit is set, and fetches only the slots those pairs need
+        auto mul_kept = [&](const half8 (&af)[H::NRB], const half8 (&bf)[4], uint32_t sb) {
+#pragma unroll
+            for (int a = 0; a < H::TRW; a++)
+#pragma unroll
+                for (int b = 0; b < G::SUB; b++) {
+                    if ((sb >> (a * G::SUB + b)) & 1u) {
+#pragma unroll
+                        for (int r = 0; r < H::RBR; r++)
+#pragma unroll
+                            for (int c = 0; c < G::RB; c++)
+                                acc[a * H::RBR + r][b * G::RB + c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                                    af[a * H::RBR + r], bf[b * G::RB + c], acc[a * H::RBR + r][b * G::RB + c], 0, 0, 0);
+                    }
+                }
+        };
+        // rows / columns of the macro tile's mask that belong to this half: needA bit a = tile row
+        // a of the half holds a kept product, needB bit b = tile column b does
+        auto need_of = [&](const u32x4 &e, uint32_t &needA, uint32_t &needB) {
+            const uint64_t m = (((uint64_t)e.w << 32) | e.z) >> (hf * H::MTA * G::MT);
+            needA = 0; needB = 0;
+#pragma unroll
+            for (int a = 0; a < H::MTA; a++) {
+                const uint32_t rowbits = (uint32_t)(m >> (a * G::MT)) & ((1u << G::MT) - 1u);
+                needA |= (rowbits ? 1u : 0u) << a;
+                needB |= rowbits;
+            }
+        };
+        uint32_t needA_tail = 0xffu, needB_tail = 0xffu;     // the stage whose head is in flight: all slots
+        const int trow0 = (hf * H::MR + wr * H::WR) / B;     // first tile row of the wave inside the macro tile
+        for (; t < S; t++) {
+            // (stages past the end repeat the last entry and are never read: their mask is cleared,
+            // so nothing is fetched for them)
+            const int tn = t + NBUF < S ? t + NBUF : S - 1;
+            u32x4 nxt = ents[tn / G::NSPE];
+            const uint32_t live = (uint32_t)((t + NBUF - S) >> 31);      // all ones while t + NBUF < S
+            nxt.z &= live;
+            nxt.w &= live;
+            SPAMM_ISSUE_N(sa_tail, needA_tail, needB_tail, 2); SPAMM_ISSUE_N(sa_tail, needA_tail, needB_tail, 3);
+            SPAMM_ISSUE_NX(sa_tail, needA_tail, needB_tail, 4); SPAMM_ISSUE_NX(sa_tail, needA_tail, needB_tail, 5);
+            const u32x4 cur = ents[t / G::NSPE];
+            const uint64_t mask = ((uint64_t)cur.w << 32) | cur.z;
+            uint32_t sb = 0;
+#pragma unroll
+            for (int a = 0; a < H::TRW; a++)
+#pragma unroll
+                for (int b = 0; b < G::SUB; b++) {
+                    const int bit = (trow0 + a) * G::MT + wc * G::SUB + b;
+                    sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
+                }
+            load_frags(a1, b1, t, 1);
+            mul_kept(a0, b0, sb);
+            sync_next();
+            sa_tail = stage_addr(t + NBUF, nxt.x);
+            need_of(nxt, needA_tail, needB_tail);
+            needA_tail = __builtin_amdgcn_readfirstlane(needA_tail);
+            needB_tail = __builtin_amdgcn_readfirstlane(needB_tail);
+            SPAMM_ISSUE_N(sa_tail, needA_tail, needB_tail, 0); SPAMM_ISSUE_N(sa_tail, needA_tail, needB_tail, 1);
+            load_frags(a0, b0, t + 1, 0);
+            mul_kept(a1, b1, sb);
+        }
+#undef SPAMM_MFMA
+#undef SPAMM_FENCE
+#undef SPAMM_LDA
+#undef SPAMM_LDB
+#undef SPAMM_ISSUE
+#undef SPAMM_ISSUE_N
+#undef SPAMM_ISSUE_X
+#undef SPAMM_ISSUE_NX
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    }
+
+    // ---- epilogue: as k_gemm's, for the half's 2 x 4 blocks per wave
+#pragma unroll
+    for (int r = 0; r < H::NRB; r++) {
+        const int64_t row0 = row_half + wr * H::WR + r * 32;
+        if (row0 >= M) continue;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int64_t col0 = (int64_t)mj * 256 + wc * 128 + c * 32;
+            if (col0 >= N) continue;
+            float *out = C + (row0 + 4 * (lane >> 5)) * N + col0 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                __builtin_nontemporal_store(acc[r][c][i], &out[(int64_t)(8 * (i / 4) + (i % 4)) * N]);
+        }
+    }
+}
+
 template <int B, int NBUF>
 static hipError_t set_lds_attr() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, NBUF>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, NBUF * GemmCfg<B>::STAGE_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, NBUF>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, NBUF * GemmCfg<B>::STAGE_BYTES);
+    if (e != hipSuccess || NBUF != HALF_RING) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_half<B, HALF_RING, 2>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, HALF_RING * HalfCfg<B, 2>::STAGE_BYTES);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_half<B, W8_RING, 4>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, W8_RING * HalfCfg<B, 4>::STAGE_BYTES);
 }
 
 hipError_t gemm_init() {
@@ -430,16 +756,28 @@ static void launch_one(unsigned grid, int n_xcd, const unsigned char *pA, const 
 }
 
 template <int B>
-static void launch_tile(int nbuf, unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB,
+static void launch_tile(int nbuf, int shape, unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB,
                         const GateBuffers &g, int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C,
                         hipStream_t s) {
+    if (shape == GEMM_SHAPE_HALF) {
+        // two workgroups per macro tile; the ring is HALF_RING stages of 24 KiB so that two workgroups fit a CU
+        k_gemm_half<B, HALF_RING, 2><<<2 * grid, 256, HALF_RING * HalfCfg<B, 2>::STAGE_BYTES, s>>>(
+            pA, pB, g.macro_list, g.macro_count, g.order, g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN, nMacN, M, N, C);
+        return;
+    }
+    if (shape == GEMM_SHAPE_W8) {
+        // a whole macro tile by eight waves of 64 x 128: two waves per SIMD
+        k_gemm_half<B, W8_RING, 4><<<grid, 512, W8_RING * HalfCfg<B, 4>::STAGE_BYTES, s>>>(
+            pA, pB, g.macro_list, g.macro_count, g.order, g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN, nMacN, M, N, C);
+        return;
+    }
     if (nbuf == 3) launch_one<B, 3>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
     else if (nbuf == 5) launch_one<B, 5>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
     else launch_one<B, 4>(grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s);
 }
 
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, hipStream_t s) {
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, int shape, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
@@ -449,9 +787,9 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
     switch (tile) {
-        case 32: launch_tile<32>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 64: launch_tile<64>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 128: launch_tile<128>(ring, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 32: launch_tile<32>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 64: launch_tile<64>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 128: launch_tile<128>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

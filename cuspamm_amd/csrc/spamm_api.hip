@@ -69,6 +69,7 @@ struct spamm_ctx : Workspace {
     int n_xcd = MAX_XCD;        // XCDs the GEMM schedule is built for (from the device's CU count)
     int gate_chunk_cap = 0;     // SPAMM_OPT_GATE_CHUNK_WORDS: the gate's k chunk, 0 = what LDS holds
     int gemm_ring = 4;          // SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's staging ring
+    int gemm_shape = 0;         // SPAMM_OPT_GEMM_SHAPE: 0 = chosen per call, else GEMM_SHAPE_FULL / GEMM_SHAPE_HALF
     uint64_t static_gen = 0;    // generation of the fixed array this context's noalloc results belong to
 
     Workspace parked;           // the workspace that is not live (see in_static)
@@ -142,6 +143,16 @@ GateBuffers gate_buffers(spamm_ctx *c) {
     g.sched = (int32_t *)c->sched.p;
     g.kept_total = (int64_t *)c->kept_total.p;
     return g;
+}
+
+// Work unit of the gated GEMM when the caller has not fixed it: with at most one macro tile per CU
+// every workgroup runs at once and the kernel's time is one workgroup's, so halves (twice the
+// workgroups, each with half the products and three quarters of the loads) finish sooner; beyond
+// that whole macro tiles by four waves are fastest (128 flop per staged byte against 85).
+int gemm_shape_for(const spamm_ctx *c) {
+    if (c->gemm_shape) return c->gemm_shape;
+    const Shape s = shape_of(c);
+    return s.n_macro <= (int64_t)c->n_xcd * SUPER_M * SUPER_N ? GEMM_SHAPE_HALF : GEMM_SHAPE_FULL;
 }
 
 int set_device(spamm_ctx *c) {
@@ -291,6 +302,10 @@ int spamm_set_option(spamm_ctx *c, int option, int value) {
             if (value < 3 || value > 5) return SPAMM_EINVAL;
             c->gemm_ring = value;
             return SPAMM_OK;
+        case SPAMM_OPT_GEMM_SHAPE:
+            if (value < 0 || value > 3) return SPAMM_EINVAL;
+            c->gemm_shape = value;
+            return SPAMM_OK;
         default:
             return SPAMM_EINVAL;
     }
@@ -433,7 +448,7 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
     HIPCHK(c, launch_gemm(c->packedA.p, c->packedB.p, gate_buffers(c), c->M, c->K, c->N, c->tile, dC,
-                          c->n_xcd, c->gemm_ring, c->stream));
+                          c->n_xcd, c->gemm_ring, gemm_shape_for(c), c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[4], c->stream)); c->ev_gemm = true; }
     return SPAMM_OK;
 }

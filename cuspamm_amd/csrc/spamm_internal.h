@@ -147,6 +147,9 @@ hipError_t launch_tau_count(const float *nA, const float *nBt, int64_t nbM, int6
 
 hipError_t gemm_init();   // one-time kernel attribute set-up
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, hipStream_t s);
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, int shape, hipStream_t s);
+// work unit of the gated GEMM: a whole macro tile (256 x 256 of C, one workgroup per CU) or half of
+// one (128 x 256, two workgroups per CU)
+constexpr int GEMM_SHAPE_FULL = 1, GEMM_SHAPE_HALF = 2, GEMM_SHAPE_W8 = 3;
 
 }  // namespace spamm

@@ -99,11 +99,16 @@ SPAMM_API int spamm_destroy(spamm_ctx *ctx);
  *   SPAMM_OPT_GATE_CHUNK_WORDS: the gate walks K in chunks of at most this many 64-k-tile bitmap
  *     words; 0 = as many as fit LDS (one chunk unless K / tile exceeds ~19 500 at tile 32).
  *   SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's operand ring, 3..5; 0 = default (4).
+ *   SPAMM_OPT_GEMM_SHAPE: work unit of the gated GEMM: 1 = a workgroup of four waves per 256 x 256
+ *     macro tile of C (one workgroup per CU), 2 = four waves per 128 x 256 half (two workgroups per
+ *     CU), 3 = eight waves per macro tile; 0 = chosen per call (halves when C has at most one macro
+ *     tile per CU, else 1).  All walk the same lists in the same order: C is bit-identical.
  * SPAMM_EINVAL for an unknown option or a value outside its range.  The reference has no such
  * knobs: its launch shapes are compile-time constants (main.h:32-73). */
 #define SPAMM_OPT_NUM_XCD 1
 #define SPAMM_OPT_GATE_CHUNK_WORDS 2
 #define SPAMM_OPT_GEMM_RING 3
+#define SPAMM_OPT_GEMM_SHAPE 4
 SPAMM_API int spamm_set_option(spamm_ctx *ctx, int option, int value);
 
 /* Run all stages on a caller-provided hipStream_t (default: the context's own

@@ -51,7 +51,7 @@ def test_option_values_match_header():
     from cuspamm_amd import api
     text = open(os.path.join(ROOT, "include", "spamm.h")).read()
     opts = dict(re.findall(r"#define\s+SPAMM_(OPT_[A-Z_]+)\s+(\d+)", text))
-    assert set(opts) == {"OPT_NUM_XCD", "OPT_GATE_CHUNK_WORDS", "OPT_GEMM_RING"}
+    assert set(opts) == {"OPT_NUM_XCD", "OPT_GATE_CHUNK_WORDS", "OPT_GEMM_RING", "OPT_GEMM_SHAPE"}
     for name, value in opts.items():
         assert getattr(api, name) == int(value), name
     L = api.load_library()

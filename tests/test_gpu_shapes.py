@@ -113,6 +113,48 @@ def test_gate_in_small_k_chunks_gives_the_same_lists(orc, ctx, chunk_words):
         other.close()
 
 
+@pytest.mark.parametrize("shape", [2, 3])
+def test_other_gemm_work_units_give_the_same_product(orc, ctx, shape):
+    """The GEMM's work unit is a whole 256 x 256 macro tile by four waves (shape 1), a 128 x 256
+    half by four waves, two workgroups per CU (2), or a whole macro tile by eight waves (3).  All
+    walk the macro tile's list in the same order, so C must agree bit for bit -- whole macro tiles,
+    ragged edges where the lower half lies beyond the matrix, all three tile sizes, dense and empty
+    regions -- and with the checker."""
+    import torch
+    import cuspamm_amd as sp
+    other = sp.SpammContext(0)
+    other.set_option(sp.OPT_GEMM_SHAPE, shape)
+    ctx.set_option(sp.OPT_GEMM_SHAPE, 1)
+    try:
+        for (M, K, N), tile, lam, ratio in [((2304, 1024, 4352), 64, 0.004, 0.3), ((1280, 512, 768), 32, 0.01, 0.5),
+                                            ((2048, 2048, 2048), 128, 0.002, 0.2), ((1024, 256, 1280), 64, 0.0, 1.0),
+                                            ((384, 2048, 320), 32, 0.003, 0.4), ((128, 1024, 128), 128, 0.0, 1.0),
+                                            ((640, 4096, 896), 128, 0.001, 0.1), ((4096, 4096, 4096), 64, 0.01, 0.05),
+                                            ((96, 64, 160), 32, 0.0, 1.0)]:
+            tab = orc.decay_table("exp", max(M, K, N), lam)
+            dA = torch.empty((M, K), dtype=torch.float32, device="cuda")
+            dB = torch.empty((K, N), dtype=torch.float32, device="cuda")
+            ctx.fill_decay(dA, tab, 1)
+            ctx.fill_decay(dB, tab, 2)
+            ctx.normmap_f32(1, dB, tile)
+            ctx.normmap_f32(0, dA, tile)
+            tau = 0.0 if ratio == 1.0 else ctx.tau_for_ratio(ratio)[0]
+            want = ctx.multiply(dA, dB, tile, tau)
+            mask, kept = ctx.get_mask(), ctx.get_stats().kept_products
+            got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            other.multiply(dA, dB, tile, tau, C=got)
+            assert np.array_equal(other.get_mask(), mask)
+            assert other.get_stats().kept_products == kept and 0 < kept
+            assert torch.equal(got, want), (M, K, N, tile)
+        tab = orc.decay_table("exp", 2048, 0.003)
+        _check(orc, other, orc.fill_decay(384, 2048, tab, 3), orc.fill_decay(2048, 320, tab, 4), 32, 0.05)
+        _check(orc, other, orc.fill_decay(640, 1024, tab, 5), orc.fill_decay(1024, 384, tab, 6), 128, 20.0)
+        _check(orc, other, orc.fill_decay(320, 1024, tab, 7), orc.fill_decay(1024, 576, tab, 8), 64, 1.0)
+    finally:
+        ctx.set_option(sp.OPT_GEMM_SHAPE, 0)
+        other.close()
+
+
 def test_scattered_sparsity_pattern(orc, ctx):
     # no band structure at all: random tiles zeroed, so k lists are ragged and macro tiles mixed
     rng = np.random.default_rng(7)
