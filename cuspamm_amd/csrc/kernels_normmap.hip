@@ -40,26 +40,23 @@ __device__ __forceinline__ float butterfly64(float v) {
     return v;
 }
 
-// One workgroup (4 waves) per strip of B rows x SW columns (SW/B tiles, SW =
-// 256: every row segment a wave reads is 1 KiB).  The tiles of a strip pass
-// through LDS in PH phases of SW/B/PH tiles each (PH = 2 for B = 128: one
-// 32 KiB tile at a time, so that three workgroups still fit a CU while their
-// loads -- all issued before the first phase -- cover the whole 256-column strip;
-// 512-byte row segments cost 4-9 % of the bandwidth).
-//   load    every wave-wide load covers 64*4/SW full strip rows, each SW*4
-//           contiguous bytes; a lane takes whole 8-row groups; all loads of a
-//           lane are in flight together.
-//   convert A role: a lane holds half a chunk (4 of 8 elements along k); the
-//           odd lane continues the even lane's running sum (DPP) so that the
-//           chunk is summed left to right.  B role: a lane holds 8 rows x 4
-//           columns and transposes in registers into 4 k-contiguous vectors.
-//   stage   fp16 vectors go to LDS in the packed tile layout (k-group
-//           segments padded by 16 bytes against bank conflicts), chunk sums
-//           to LDS at their canonical index.
-//   store   after one barrier: the tiles are copied out with contiguous 1 KiB
-//           wave stores (a packed tile is one contiguous block in memory), and
-//           one wave per tile applies the canonical reduction.
-// (The phased A role is held to three waves per SIMD: it gains more from a third resident
+// One workgroup (4 waves) per strip of B rows x SW columns (SW/B tiles; SW = 256 for fp32 input,
+// 512 for fp16 input: a strip row is 1 KiB either way and is read by one wave-wide load).  The
+// tiles of a strip pass through LDS in PH phases of SW/B/PH tiles each, sized so that at most
+// ~42 KiB are resident and three workgroups fit a CU; all loads are issued before the first phase.
+//   load    a lane takes whole 8-row groups (wave w: groups w, w + 4, ...); all loads of a lane
+//           are in flight together.
+//   convert fp32 input, A role: a lane holds half a chunk (4 of 8 elements along k); the odd lane
+//           continues the even lane's running sum (DPP) so that the chunk is summed left to
+//           right.  B role: a lane holds 8 rows x 4 columns and transposes in registers into 4
+//           k-contiguous vectors.  fp16 input: a lane's 16 bytes are a whole chunk (A role) or,
+//           over 8 rows, an 8 x 8 block transposed in registers (B role).
+//   stage   fp16 vectors go to LDS in the packed tile layout (k-group segments padded by 16
+//           bytes against bank conflicts), chunk sums to LDS at their canonical index.
+//   store   after one barrier: the tiles are copied out with contiguous 1 KiB wave stores (a
+//           packed tile is one contiguous block in memory), and one wave per tile applies the
+//           canonical reduction.
+// (The phased fp32 A role is held to three waves per SIMD: it gains more from a third resident
 // workgroup than it loses to a few spilled registers; the B role would spill far more.)
 template <int B, int ROLE, int SW, bool IN16, int PH = 1>
 __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
@@ -71,21 +68,15 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k
     constexpr int TPS = SW / B;           // tiles per strip
     constexpr int TPP = TPS / PH;         // tiles per phase (resident in LDS together)
     static_assert(TPP * PH == TPS && TPP >= 1, "phases must divide the strip's tiles");
-    // Lane -> element mapping.
-    // fp32 input, PH = 1: a wave-wide load covers whole strip rows (LPR lanes each, 4 columns a
-    // lane).  PH > 1: the waves are split between the phases' tiles (WPP waves per phase), a
-    // wave-wide load covers rows of its own tiles only (the waves of the other phases read the
-    // neighbouring segments of the same rows at the same time), and a phase is staged by whole
-    // waves.
-    // fp16 input (IN16): a lane takes 8 columns (16 bytes), the strip is 512 columns wide and every
-    // wave-wide load is one whole strip row (1 KiB) whatever PH is; a lane's columns lie in one
-    // tile, and in phase ph only the lanes of that phase's tiles stage their data.
+    // Lane -> element mapping: every wave-wide load is one whole strip row (1 KiB): 64 lanes x EPL
+    // columns (4 floats, or 8 halves for fp16 input: the strip is then 512 columns wide); wave w
+    // takes the 8-row groups w, w + 4, ...  A lane's columns lie in one tile; with PH > 1 the tiles
+    // pass through LDS PH phases one after the other and in phase ph only the lanes of that
+    // phase's tiles stage their data.  (Tile 128 used to split the waves between its two tiles at
+    // load time -- 512-byte row segments -- which measured 0-4 % slower than whole rows.)
     constexpr int EPL = IN16 ? 8 : 4;                  // columns per lane
-    static_assert(!IN16 || SW == 512, "fp16 input: 64 lanes x 8 columns");
-    constexpr int WPP = IN16 ? 4 : 4 / PH;             // waves that share a row range
-    constexpr int LPR = IN16 ? 64 : (PH > 1 ? TPP * B : SW) / 4;   // lanes across one row of the wave's columns
-    constexpr int RH = 64 / LPR;                       // rows per wave-wide load
-    constexpr int GSTEP = WPP * RH;                    // 8-row groups between a lane's groups
+    static_assert(SW == 64 * EPL, "a strip row is one wave-wide load");
+    constexpr int GSTEP = 4;                           // 8-row groups between a lane's groups (one per wave)
     static_assert(PH == 1 || PH == 2 || PH == 4, "phases are made of whole waves");
     constexpr int QN = B / 8;             // k-groups per tile
     constexpr int VPT = B * B / 8;        // 16-byte vectors per tile
@@ -103,8 +94,8 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k
     const int64_t I = blockIdx.x / nstrip;            // tile row of the strip
     const int64_t sc = blockIdx.x % nstrip;
     const int64_t col0 = sc * SW;
-    const int cl = IN16 ? EPL * lane : (wave / WPP) * (TPP * B) + 4 * (lane % LPR);   // first column of this lane inside the strip
-    const int g0 = (wave % WPP) * RH + lane / LPR;    // first 8-row group of this lane; then every GSTEP-th
+    const int cl = EPL * lane;                        // first column of this lane inside the strip
+    const int g0 = wave;                              // first 8-row group of this lane; then every GSTEP-th
     const int t = cl / B, cin = cl % B;               // tile of the strip, column inside the tile
     const bool valid = col0 + cl < cols;
     const int64_t eoff = (I * B) * ld + col0 + cl;
