@@ -88,6 +88,38 @@ def measured_trace_us(workload, profile_dir=PROFILE_DIR):
     return out
 
 
+def gemm_structure(ctx, N, tile, kept, n_cu=256, cu_per_xcd=32):
+    """Shape of the GEMM's work from the gate's own lists: how many macro tiles (256 x 256 of C) hold
+    work, how they fall on the CUs, how much of the k loop runs kept-by-all ("full") stages, how
+    full the others are, and how much of C is only zero-filled."""
+    counts, sched = ctx.get_macro_counts()
+    U, F = counts[..., 0].astype(np.int64), counts[..., 1].astype(np.int64)
+    mt = 256 // tile                                  # output tiles per macro tile per dimension
+    nspe = tile // 32                                 # 32-k stages per list entry
+    computing = int((U > 0).sum())
+    n_xcd = max(1, n_cu // cu_per_xcd)
+    per_xcd = [int(v) for v in sched[:n_xcd]]
+    stages, full_stages = int(U.sum()) * nspe, int(F.sum()) * nspe
+    partial_entries = int((U - F).sum())
+    kept_in_full = int(F.sum()) * mt * mt
+    rounds_mean = computing / n_cu
+    rounds_max = max(-(-v // cu_per_xcd) for v in per_xcd) if per_xcd else 0
+    lens = U[U > 0]
+    return {
+        "macro_tiles": int(U.size), "computing_macro_tiles": computing, "empty_macro_tiles": int(U.size) - computing,
+        "computing_per_xcd": per_xcd,
+        "rounds_per_cu_mean": round(rounds_mean, 3), "rounds_per_cu_max": rounds_max,
+        "round_quantisation_loss": round(1.0 - rounds_mean / rounds_max, 4) if rounds_max else None,
+        "list_length_entries": {"mean": round(float(lens.mean()), 1) if lens.size else 0.0,
+                                "min": int(lens.min()) if lens.size else 0, "max": int(lens.max()) if lens.size else 0},
+        "stages": stages, "full_stage_share": round(full_stages / stages, 4) if stages else None,
+        "partial_stage_share": round(1.0 - full_stages / stages, 4) if stages else None,
+        "partial_stage_fill": (round((kept - kept_in_full) / (partial_entries * mt * mt), 4) if partial_entries else None),
+        "zero_fill_bytes": (int(U.size) - computing) * 256 * 256 * 4,
+        "zero_fill_share_of_c": round(1.0 - computing / U.size, 4),
+    }
+
+
 def decay_table(kind, n, lam):
     d = np.arange(n, dtype=np.float64)
     if kind == "exp":
@@ -163,6 +195,10 @@ def main():
                          "error report, literal config or CPU baseline")
     ap.add_argument("--skip-variants", action="store_true",
                     help="skip the fp16-input / REUSE_B / A_EQ_B / no-prune timings")
+    ap.add_argument("--calibrate-cache", action="store_true",
+                    help="only run the read-only reference kernels of the dev library: 4 GiB streamed from HBM and a 96 MiB "
+                         "buffer re-read from the memory-side cache, each with a full grid and with 32 workgroups: "
+                         "reference points for the L2-miss read latency (TCC_EA0_RDREQ_LEVEL / TCC_EA0_RDREQ)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (reference point for FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -184,6 +220,12 @@ def main():
             y.copy_(x)
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": x.numel() * 4, "bytes_written": x.numel() * 4, "launches": 5}))
+        return
+
+    if args.calibrate_cache:
+        from cuspamm_amd import dev as spdev
+        names = ("hbm_stream_full_grid", "cache_reread_full_grid", "hbm_stream_32_workgroups", "cache_reread_32_workgroups")
+        print(json.dumps({"calibrate_cache_GBps": {n: round(spdev.read_reference(0, i), 1) for i, n in enumerate(names)}}))
         return
 
     if args.skip_extras:
@@ -265,6 +307,7 @@ def main():
     b_tiles_read = int(np.unpackbits(b_need.view(np.uint8)).sum())
     del gm
     gemm_alg_bytes = 4.0 * N * N + 2.0 * tile * tile * (a_tiles_read + b_tiles_read)
+    structure = gemm_structure(ctx, N, tile, kept)
     trace_us = measured_trace_us(args.workload)
     nm_gbs = nm_bytes_b / (stage[0] * 1e-3) / 1e9                      # the B pass
 
@@ -291,6 +334,7 @@ def main():
         },
         "stage_ms": {"normmap_b": round(stage[0], 4), "normmap_a": round(stage[1], 4), "gate": round(stage[2], 4),
                      "gemm": round(stage[3], 4), "sum_events": round(stage[4], 4)},
+        "gemm_structure": structure,
         "gemm_only_tflops": round(gemm_tflops, 2),
         "gemm_only_frac_of_fp16_peak": round(gemm_tflops / PEAK_FP16_TFLOPS, 4),
         "whole_multiply_frac_of_fp16_peak": round(value / PEAK_FP16_TFLOPS, 4),

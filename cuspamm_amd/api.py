@@ -95,6 +95,7 @@ def load_library():
     L.spamm_get_klist.argtypes = [vp, vp]
     L.spamm_get_mask.argtypes = [vp, vp]
     L.spamm_get_fp16.argtypes = [vp, ctypes.c_int, vp]
+    L.spamm_get_macro_counts.argtypes = [vp, vp, vp]
     L.spamm_get_stats.argtypes = [vp, ctypes.POINTER(SpammStats)]
     L.spamm_fill_decay_f32.argtypes = [vp, vp, i64, i64, vp, ctypes.c_uint64, ctypes.c_int]
     L.spamm_synchronize.argtypes = [vp]
@@ -346,6 +347,15 @@ class SpammContext:
         out = np.empty((nbM, nbN, (nbK + 63) // 64), dtype=np.uint64)
         _check(self._lib.spamm_get_mask(self._h, out.ctypes.data), "spamm_get_mask")
         return out
+
+    def get_macro_counts(self):
+        """(counts [macro rows, macro columns, 2] = list length / kept-by-all entries per 256 x 256 macro
+        tile of C, sched [16] = per XCD macro tiles with work, then all macro tiles)."""
+        M, N = self._shape[4], self._shape[6]
+        counts = np.empty(((M + 255) // 256, (N + 255) // 256, 2), dtype=np.int32)
+        sched = np.empty(16, dtype=np.int32)
+        _check(self._lib.spamm_get_macro_counts(self._h, counts.ctypes.data, sched.ctypes.data), "spamm_get_macro_counts")
+        return counts, sched
 
     def get_fp16(self, role):
         M, K, N = self._shape[4:7]

@@ -873,6 +873,16 @@ int spamm_get_mask(spamm_ctx *c, uint64_t *host_out) {
     return copy_out(c, c->mask.p, host_out, (size_t)s.nbM * s.nbN * s.words * 8);
 }
 
+int spamm_get_macro_counts(spamm_ctx *c, int32_t *host_counts, int32_t *host_sched) {
+    if (!c || !host_counts) return SPAMM_EINVAL;
+    if (static_stale(c)) return SPAMM_ESTATE;
+    if (!c->have_gate) return SPAMM_ESTATE;
+    const Shape s = shape_of(c);
+    int rc = copy_out(c, c->macro_count.p, host_counts, (size_t)s.n_macro * 8);
+    if (rc == SPAMM_OK && host_sched) rc = copy_out(c, c->sched.p, host_sched, 2 * MAX_XCD * 4);
+    return rc;
+}
+
 int spamm_get_fp16(spamm_ctx *c, int role, uint16_t *host_out) {
     if (!c || !host_out) return SPAMM_EINVAL;
     if (static_stale(c)) return SPAMM_ESTATE;

@@ -17,8 +17,18 @@ def load_dev_library():
         L = ctypes.CDLL(DEV_LIB_PATH)
         L.spamm_dev_mfma_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                              ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+        L.spamm_dev_read_reference.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
         _lib = L
     return _lib
+
+
+def read_reference(device=0, which=0):
+    """GB/s of one of the four read-only reference kernels (see include/spamm_dev.h)."""
+    g = ctypes.c_double(0)
+    rc = load_dev_library().spamm_dev_read_reference(int(device), int(which), ctypes.byref(g))
+    if rc != 0:
+        raise RuntimeError("spamm_dev_read_reference failed: %d" % rc)
+    return float(g.value)
 
 
 def mfma_ceiling(device=0, random_operands=True, iters=20000):

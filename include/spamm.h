@@ -209,6 +209,13 @@ SPAMM_API int spamm_get_counts(spamm_ctx *ctx, int32_t *host_out);
 SPAMM_API int spamm_get_klist(spamm_ctx *ctx, uint16_t *host_out);
 SPAMM_API int spamm_get_mask(spamm_ctx *ctx, uint64_t *host_out);
 SPAMM_API int spamm_get_fp16(spamm_ctx *ctx, int role, uint16_t *host_out);
+/* The work list the gate built for the GEMM (the reference has none: every block re-gates its own
+ * tile, cuSpAMM.cu:302-334): per macro tile of C (256 x 256 elements, row-major over
+ * ceil(M/256) x ceil(N/256)) host_counts[2 m] = k tiles kept by at least one of its output tiles
+ * (the length of the list its workgroup walks), host_counts[2 m + 1] = of which kept by all of
+ * them; host_sched (optional, 16 ints): per XCD x the number of macro tiles with work [x] and of
+ * all macro tiles [8 + x] in its sequence. */
+SPAMM_API int spamm_get_macro_counts(spamm_ctx *ctx, int32_t *host_counts, int32_t *host_sched);
 
 /* Synchronises and fills `out` (kept-product count as in countValid,
  * tool.cu:493-529; per-stage times replace the whole-iteration cudaEvent pair,

@@ -32,6 +32,14 @@ extern "C" {
 SPAMM_DEV_API int spamm_dev_mfma_ceiling(int device, int random_operands, int iters, double *tflops,
                                          double *clock_ghz);
 
+/* Read-only reference kernels for reading cache counters of other kernels against: `which` = 0: one
+ * pass over 4 GiB with a full grid (every read comes from HBM, queues full); 1: 40 passes over one
+ * 96 MiB buffer (misses the 4 MB L2s, stays in the 256 MB memory-side cache); 2 and 3: the same two
+ * with 32 workgroups (idle queues: latency rather than bandwidth).  Each runs three times; *gbps is
+ * the best.  Kernel names k_dev_read<which> tell them apart in a profile.  Returns 0 or the negative
+ * of the failing hipError_t (-1 for bad arguments). */
+SPAMM_DEV_API int spamm_dev_read_reference(int device, int which, double *gbps);
+
 #ifdef __cplusplus
 }
 #endif

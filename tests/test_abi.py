@@ -38,12 +38,13 @@ def test_dev_library_is_separate_from_the_engine():
     from cuspamm_amd import dev
     text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "spamm_dev.h")).read(), flags=re.S)
     syms = sorted(set(re.findall(r"\b(spamm_dev_[a-z0-9_]+)\s*\(", text)))
-    assert syms == ["spamm_dev_mfma_ceiling"]
+    assert syms == ["spamm_dev_mfma_ceiling", "spamm_dev_read_reference"]
     D = dev.load_dev_library()
     for name in syms:
         assert hasattr(D, name), name
     L = sp.load_library()
     assert not hasattr(L, "spamm_mfma_ceiling") and not hasattr(L, "spamm_dev_mfma_ceiling")
+    assert D.spamm_dev_read_reference(0, 9, None) == -1
     assert D.spamm_dev_mfma_ceiling(0, 0, 0, None, None) == -1        # bad arguments: refused before any device call
 
 

@@ -84,6 +84,34 @@ def test_multiply_matches_checker(orc, ctx, M, K, N, tile, kind, lam, tau):
         assert 0 < ref["kept"] < total, "case does not exercise the gate"
 
 
+@pytest.mark.parametrize("M,K,N,tile,lam,tau", [(1024, 2048, 768, 64, 0.004, 0.3), (640, 1024, 896, 32, 0.01, 0.05),
+                                                 (512, 4096, 1280, 128, 0.002, 5.0)])
+def test_macro_tile_work_lists_match_the_mask(orc, ctx, M, K, N, tile, lam, tau):
+    """spamm_get_macro_counts against the checker's mask: per 256 x 256 macro tile of C the number of
+    k tiles kept by any of its output tiles and by all of them, and the per-XCD totals."""
+    tab = orc.decay_table("exp", max(M, K, N), lam)
+    A, B = orc.fill_decay(M, K, tab, 1), orc.fill_decay(K, N, tab, 2)
+    ctx.multiply(_dev(A), _dev(B), tile, tau)
+    ref = orc.spamm(A, B, tile, tau)
+    counts, sched = ctx.get_macro_counts()
+    nbM, nbK, nbN, mt = M // tile, K // tile, N // tile, 256 // tile
+    bits = np.unpackbits(ref["mask"].view(np.uint8), axis=2, bitorder="little")[:, :, :nbK].astype(bool)   # [i, j, k]
+    want = np.zeros_like(counts)
+    for mi in range(counts.shape[0]):
+        for mj in range(counts.shape[1]):
+            blk = bits[mi * mt:(mi + 1) * mt, mj * mt:(mj + 1) * mt].reshape(-1, nbK)
+            want[mi, mj, 0] = np.count_nonzero(blk.any(axis=0))
+            # "kept by all" counts the tiles inside the matrix only when the macro tile is whole
+            want[mi, mj, 1] = np.count_nonzero(blk.all(axis=0)) if blk.shape[0] == mt * mt else 0
+    assert np.array_equal(counts[..., 0], want[..., 0])
+    whole = np.zeros(counts.shape[:2], dtype=bool)
+    whole[:nbM // mt, :nbN // mt] = True
+    assert np.array_equal(counts[..., 1][whole], want[..., 1][whole])
+    assert np.all(counts[..., 1] <= counts[..., 0])
+    assert 0 < np.count_nonzero(counts[..., 0]) and sched[:8].sum() == np.count_nonzero(counts[..., 0])
+    assert sched[8:].sum() == counts.shape[0] * counts.shape[1]
+
+
 def test_baseline_config1_a_equals_b(orc, ctx):
     # N=1024, A=B, exp(-0.5|i-j|), tile 32, tau=1e-4
     tab = orc.decay_table("exp", 1024, 0.5)
