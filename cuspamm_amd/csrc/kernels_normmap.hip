@@ -58,8 +58,8 @@ __device__ __forceinline__ float butterfly64(float v) {
 //           canonical reduction.
 // (The phased fp32 A role is held to three waves per SIMD: it gains more from a third resident
 // workgroup than it loses to a few spilled registers; the B role would spill far more.)
-template <int B, int ROLE, int SW, bool IN16, int PH = 1>
-__global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
+template <int B, int ROLE, int SW, bool IN16, int PH = 1, int NWV = 4>
+__global__ __launch_bounds__(64 * NWV, (PH > 1 && ROLE == 0 && !IN16 && NWV == 4) ? 3 : 1) void k_normmap(const void *__restrict__ Xv, int64_t ld, int64_t cols,
                                                  int64_t nbr, int64_t nbc, int64_t nstrip,
                                                  uint4 *__restrict__ packed, float *__restrict__ nm,
                                                  float *__restrict__ nmT, uint4 *__restrict__ packed2,
@@ -76,7 +76,8 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k
     // load time -- 512-byte row segments -- which measured 0-4 % slower than whole rows.)
     constexpr int EPL = IN16 ? 8 : 4;                  // columns per lane
     static_assert(SW == 64 * EPL, "a strip row is one wave-wide load");
-    constexpr int GSTEP = 4;                           // 8-row groups between a lane's groups (one per wave)
+    constexpr int GSTEP = NWV;                         // 8-row groups between a lane's groups (one per wave)
+    static_assert(B % (8 * NWV) == 0, "every wave takes whole 8-row groups");
     static_assert(PH == 1 || PH == 2 || PH == 4, "phases are made of whole waves");
     constexpr int QN = B / 8;             // k-groups per tile
     constexpr int VPT = B * B / 8;        // 16-byte vectors per tile
@@ -247,8 +248,8 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k
     __shared__ int s_skip[TPP];
     auto copy_out = [&](int ph, bool as_b, uint4 *__restrict__ pk, bool prune) {
 #pragma unroll
-        for (int i = 0; i < TPP * VPT / 256; i++) {
-            const int vi = threadIdx.x + 256 * i;
+        for (int i = 0; i < TPP * VPT / (64 * NWV); i++) {
+            const int vi = threadIdx.x + 64 * NWV * i;
             const int tt = vi / VPT, iv = vi % VPT;
             const int64_t Jt = sc * TPS + ph * TPP + tt;
             if (Jt < nbc && !(prune && s_skip[tt])) {
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(256, (PH > 1 && ROLE == 0 && !IN16) ? 3 : 1) void k
     // bound is max_j nB[k,j] for the A pass (B's norm map is complete by then) and the largest
     // finite float for the B pass, which runs first: there only tiles of norm zero are left out.
     auto norms = [&](int ph, bool as_b, float *__restrict__ nmo, float *__restrict__ nmTo, bool prune) {
-        for (int tt = wave; tt < TPP; tt += 4) {
+        for (int tt = wave; tt < TPP; tt += NWV) {
             const int64_t Jt = sc * TPS + ph * TPP + tt;
             if (Jt >= nbc) break;
             const float rmax = prune ? (rowmax != nullptr ? rowmax[Jt] : 3.402823466e+38f) : 0.0f;
@@ -410,7 +411,16 @@ static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int 
     switch (tile) {
         case 32: k_normmap<32, ROLE, SW, IN16, 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         case 64: k_normmap<64, ROLE, SW, IN16, IN16 ? 2 : 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
-        case 128: k_normmap<128, ROLE, SW, IN16, IN16 ? 4 : 2><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        // tile 128: eight waves per workgroup (two 8-row groups per lane instead of four: no register
+        // spills, more loads in flight) where that measured faster -- the fp32 A role (3.36 -> 3.07 ms at
+        // N = 65536) and both roles on fp16 input (2.02 -> 1.85, 1.95 -> 1.90 ms) -- but not the fp32 B
+        // role (3.26 -> 3.93 ms) nor, by extension, the single pass for A = B
+        case 128:
+            if constexpr (IN16 || ROLE == 0) {
+                k_normmap<128, ROLE, SW, IN16, IN16 ? 4 : 2, 8><<<grid, 512, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip);
+                break;
+            }
+            k_normmap<128, ROLE, SW, IN16, IN16 ? 4 : 2><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
