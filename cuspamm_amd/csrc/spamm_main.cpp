@@ -10,7 +10,10 @@
 //
 //   spamm_main [--M m] [--K k] [--N n] [--tile 32|64|128] [--tau t | --ratio r | --tune r]
 //              [--gen exp|alg|ones] [--c c] [--v v] [--a-csv f --b-csv f | --a-mtx f --b-mtx f]
-//              [--testtime n] [--warmup n] [--check | --prune] [--noalloc] [--device d]
+//              [--testtime n] [--warmup n] [--check | --prune] [--noalloc | --half] [--device d]
+// --half: the operands are rounded to fp16 on the host and resident as fp16 before the timed
+// multiplies, as in the reference (USINGHALF 1, para.h:1; __float2half in its generators,
+// tool.cu:418,432); without it the fp32 -> fp16 conversion is part of every timed multiply.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -37,7 +40,7 @@ int main(int argc, char **argv) {
     bool cv_given = false;
     std::string a_csv, b_csv, a_mtx, b_mtx;
     int testtime = 10, warmup = 5, device = 0;         // TESTTIME, WARMUP, para.h:4-5
-    bool check = false, prune = false, noalloc = false;
+    bool check = false, prune = false, noalloc = false, half_in = false;
     for (int i = 1; i < argc; i++) {
         const std::string o = argv[i];
         auto val = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };
@@ -60,12 +63,14 @@ int main(int argc, char **argv) {
         else if (o == "--device") device = atoi(val());
         else if (o == "--check") check = true;
         else if (o == "--prune") prune = true;
+        else if (o == "--half") half_in = true;
         else if (o == "--noalloc") noalloc = true;        // the timed multiplies run in the library's fixed workspace
         else { fprintf(stderr, "spamm_main: unknown option %s\n", o.c_str()); return 2; }
     }
     if (gen == "exp" && !cv_given) { c = 1.0f; v = 0.1f; }    // getDecayMatrixExp(h, 1, 0.1, ...), cuSpAMM.cu:426-427
     if (tile != 32 && tile != 64 && tile != 128) { fprintf(stderr, "spamm_main: tile must be 32, 64 or 128\n"); return 2; }
     if (check && prune) { fprintf(stderr, "spamm_main: --check needs A's complete fp16 copy, --prune leaves tiles out\n"); return 2; }
+    if (half_in && noalloc) { fprintf(stderr, "spamm_main: --noalloc takes fp32 operands, not --half\n"); return 2; }
     if (inM <= 0 || inK <= 0 || inN <= 0 || testtime <= warmup + 1) { fprintf(stderr, "spamm_main: bad sizes\n"); return 2; }
     // padded dimensions (main.h:54-56)
     const long long M = (inM + tile - 1) / tile * tile, K = (inK + tile - 1) / tile * tile, N = (inN + tile - 1) / tile * tile;
@@ -123,12 +128,29 @@ int main(int argc, char **argv) {
         p.tau = tau;
     }
 
+    void *dAh = nullptr, *dBh = nullptr;
+    if (half_in) {
+        // host-side rounding to fp16 (round to nearest even, what __float2half does), then upload
+        auto to_half = [&](const float *dsrc, size_t n, void **dst) -> bool {
+            std::vector<float> h32(n);
+            std::vector<_Float16> h16(n);
+            if (hipMemcpy(h32.data(), dsrc, n * 4, hipMemcpyDeviceToHost) != hipSuccess) return false;
+            for (size_t i = 0; i < n; i++) h16[i] = (_Float16)h32[i];
+            return hipMalloc(dst, n * 2) == hipSuccess && hipMemcpy(*dst, h16.data(), n * 2, hipMemcpyHostToDevice) == hipSuccess;
+        };
+        if (!to_half(dA, (size_t)M * K, &dAh) || !to_half(dB, (size_t)K * N, &dBh)) {
+            fprintf(stderr, "spamm_main: fp16 copies of the operands failed\n");
+            return 1;
+        }
+    }
+
     double sum = 0.0;
     spamm_stats st;
     memset(&st, 0, sizeof(st));
     for (int i = 0; i < testtime; i++) {
-        if ((rc = noalloc ? spamm_multiply_noalloc(ctx, &p, dA, dB, dC) : spamm_multiply(ctx, &p, dA, dB, dC)))
-            return fail(noalloc ? "spamm_multiply_noalloc" : "spamm_multiply", rc);
+        if ((rc = half_in ? spamm_multiply_f16(ctx, &p, dAh, dBh, dC)
+                          : (noalloc ? spamm_multiply_noalloc(ctx, &p, dA, dB, dC) : spamm_multiply(ctx, &p, dA, dB, dC))))
+            return fail(half_in ? "spamm_multiply_f16" : (noalloc ? "spamm_multiply_noalloc" : "spamm_multiply"), rc);
         if ((rc = spamm_get_stats(ctx, &st))) return fail("spamm_get_stats", rc);
         if (i > warmup) sum += st.ms_total * 1e-3;       // cuSpAMM.cu:548
     }
@@ -145,6 +167,8 @@ int main(int argc, char **argv) {
         // the reference prints ||C_dense - C||_F, ||C_dense||_F, ||C||_F (tool.cu:270-276)
         printf("error check: |C_dense-C|_F=%e |C_dense|_F=%e |C|_F=%e bound=%e\n", e3[0], e3[1], e3[2], bound);
     }
+    if (dAh) (void)hipFree(dAh);
+    if (dBh) (void)hipFree(dBh);
     (void)hipFree(dA);
     (void)hipFree(dB);
     (void)hipFree(dC);

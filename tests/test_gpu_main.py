@@ -54,6 +54,24 @@ def test_driver_pads_and_tunes(orc):
     assert total == 16 * 15 * 18 and abs(ach - 0.3) < 0.02 and abs(kept / total - ach) < 1e-6
 
 
+def test_driver_defaults_are_the_reference_experiment_with_fp16_operands(orc):
+    # no options: 2048^3, tile 32, getDecayMatrixAlg(0.1, 0.1), Norm = 1.548969 (para.h:1-14, cuSpAMM.cu:428-431);
+    # --half: the operands are fp16 before the timed multiplies, as USINGHALF 1 has them
+    plain, half = _run(["--check"]), _run(["--half", "--check"])
+    for out in (plain, half):
+        assert "input parameters: M=2048 K=2048 N=2048 Norm=1.548969" in out
+    pick = lambda out: (re.search(r"valid products=(\d+) of (\d+)", out).groups(),
+                        re.search(r"\|C_dense-C\|_F=(\S+) \|C_dense\|_F=(\S+) \|C\|_F=(\S+) bound=(\S+)", out).groups())
+    assert pick(plain) == pick(half)            # rounding to fp16 on the host or on the device: the same operands
+    kept, total = map(int, pick(half)[0])
+    tab = orc.decay_table("ref_alg", 2048, c=0.1, v=0.1)
+    A = orc.fill_decay(2048, 2048, tab, 0, random=False)
+    ref = orc.spamm(A, A, 32, 1.548969)
+    assert total == 64 ** 3 and abs(kept - ref["kept"]) <= max(2, ref["kept"] // 1000)
+    proc = subprocess.run([MAIN, "--half", "--noalloc"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert proc.returncode == 2 and "--half" in proc.stdout
+
+
 def test_driver_rejects_bad_arguments():
     proc = subprocess.run([MAIN, "--tile", "48"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     assert proc.returncode == 2 and "tile must be" in proc.stdout
