@@ -41,8 +41,9 @@ extern "C" {
 #define SPAMM_ROLE_B 1       /* contraction along rows:    B[K x N] */
 
 /* spamm_params.flags */
-#define SPAMM_FLAG_A_EQ_B 1u     /* dA == dB, M == K == N: the matrix is read once for both operand roles
-                                  * (else SPAMM_EINVAL); the single pass is reported as ms_normmap_b */
+#define SPAMM_FLAG_A_EQ_B 1u     /* dA == dB, M == K == N (else SPAMM_EINVAL): at tile 32 and 64 the matrix is read once
+                                  * for both operand roles (the single pass is reported as ms_normmap_b); at tile 128
+                                  * the two ordinary passes run (they are faster there) */
 #define SPAMM_FLAG_TIMING 2u     /* record per-stage HIP events (spamm_get_stats) */
 #define SPAMM_FLAG_REUSE_A 4u    /* A's fp16 copy and norm map from an earlier call are reused (dA ignored) */
 #define SPAMM_FLAG_REUSE_B 8u    /* same for B: e.g. one B against many A, or matrix powers */
