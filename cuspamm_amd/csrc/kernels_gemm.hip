@@ -404,21 +404,22 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 
 
 // ---------------------------------------------------------------------------
-// The same multiply with a workgroup per HALF macro tile: 128 rows x 256 columns of C, 4 waves
-// (2 x 2), each wave 64 x 128 = 2 x 4 MFMA blocks = 128 accumulator registers, so two workgroups
-// (two waves per SIMD) share a CU: one workgroup's prologue, epilogue, barriers and LDS reads sit
-// under the other's MFMAs, and the work units are half as long (finer tail).  The price is the B
-// part of a stage staged once per half: 24 KiB per 2.1 Mflop instead of 32 KiB per 4.2 Mflop.
+// k_gemm_w64: the same multiply by waves of 64 x 128 (2 x 4 MFMA blocks = 128 accumulator
+// registers, two waves per SIMD), NWR wave rows x 2 wave columns per workgroup:
+//   NWR = 2  a workgroup per HALF macro tile (128 x 256 of C), two workgroups per CU: one's
+//            prologue, epilogue, barriers and LDS reads sit under the other's MFMAs and the work
+//            units are half as long (finer tail); the price is the B part of a stage staged once
+//            per half, 24 KiB per 2.1 Mflop instead of 32 KiB per 4.2 Mflop.  Workgroups 2 q and
+//            2 q + 1 of an XCD's sequence take the upper and lower half of its q-th macro tile.
+//   NWR = 4  a whole macro tile by eight waves: k_gemm's 32 KiB per stage, two waves per SIMD.
 // Lists, masks and the order of accumulation are the macro tile's, so C is bit-identical to
-// k_gemm's.  Workgroup pair (2 q, 2 q + 1) of an XCD's sequence takes the upper and lower half of
-// the XCD's q-th macro tile.
+// k_gemm's.  Measured against k_gemm: halves lose 7-12 % where there is much work per CU and win
+// where there is at most one macro tile per CU (chosen there); eight waves are within 1-3 %.
 constexpr int HALF_RING = 3;      // stages of the half shape's ring: 3 x 24 KiB, two workgroups per CU
 constexpr int W8_RING = 4;        // stages of the eight-wave shape's ring: 4 x 32 KiB, one workgroup per CU
 
-// NWR wave rows of 64 rows of C each: 2 = the half shape above, 4 = a whole macro tile by eight
-// waves (4 x 2; the same 32 KiB per stage as k_gemm, but two waves per SIMD).
 template <int B, int NWR>
-struct HalfCfg {
+struct W64Cfg {
     using G = GemmCfg<B>;
     static constexpr int NW = 2 * NWR;                       // waves per workgroup
     static constexpr int MR = 64 * NWR, WR = 64, NRB = 2;
@@ -438,7 +439,7 @@ struct HalfCfg {
 };
 
 template <int B, int NBUF, int NWR>
-__global__ __launch_bounds__(128 * NWR, NWR == 2 ? 2 : 1) void k_gemm_half(const unsigned char *__restrict__ pA,
+__global__ __launch_bounds__(128 * NWR, NWR == 2 ? 2 : 1) void k_gemm_w64(const unsigned char *__restrict__ pA,
                                                       const unsigned char *__restrict__ pB,
                                                       const MacroEntry *__restrict__ macro_list,
                                                       const int32_t *__restrict__ macro_count,
@@ -447,7 +448,7 @@ __global__ __launch_bounds__(128 * NWR, NWR == 2 ? 2 : 1) void k_gemm_half(const
                                                       int nbK, int nbN, int nMacN, int64_t M, int64_t N,
                                                       float *__restrict__ C) {
     using G = GemmCfg<B>;
-    using H = HalfCfg<B, NWR>;
+    using H = W64Cfg<B, NWR>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef const __attribute__((address_space(4))) u32x4 *entry_ptr;   // scalar (SMEM) loads
 
@@ -726,11 +727,11 @@ static hipError_t set_lds_attr() {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, NBUF>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, NBUF * GemmCfg<B>::STAGE_BYTES);
     if (e != hipSuccess || NBUF != HALF_RING) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_half<B, HALF_RING, 2>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, HALF_RING * HalfCfg<B, 2>::STAGE_BYTES);
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_w64<B, HALF_RING, 2>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, HALF_RING * W64Cfg<B, 2>::STAGE_BYTES);
     if (e != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_half<B, W8_RING, 4>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, W8_RING * HalfCfg<B, 4>::STAGE_BYTES);
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_w64<B, W8_RING, 4>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, W8_RING * W64Cfg<B, 4>::STAGE_BYTES);
 }
 
 hipError_t gemm_init() {
@@ -761,13 +762,13 @@ static void launch_tile(int nbuf, int shape, unsigned grid, int n_xcd, const uns
                         hipStream_t s) {
     if (shape == GEMM_SHAPE_HALF) {
         // two workgroups per macro tile; the ring is HALF_RING stages of 24 KiB so that two workgroups fit a CU
-        k_gemm_half<B, HALF_RING, 2><<<2 * grid, 256, HALF_RING * HalfCfg<B, 2>::STAGE_BYTES, s>>>(
+        k_gemm_w64<B, HALF_RING, 2><<<2 * grid, 256, HALF_RING * W64Cfg<B, 2>::STAGE_BYTES, s>>>(
             pA, pB, g.macro_list, g.macro_count, g.order, g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN, nMacN, M, N, C);
         return;
     }
     if (shape == GEMM_SHAPE_W8) {
         // a whole macro tile by eight waves of 64 x 128: two waves per SIMD
-        k_gemm_half<B, W8_RING, 4><<<grid, 512, W8_RING * HalfCfg<B, 4>::STAGE_BYTES, s>>>(
+        k_gemm_w64<B, W8_RING, 4><<<grid, 512, W8_RING * W64Cfg<B, 4>::STAGE_BYTES, s>>>(
             pA, pB, g.macro_list, g.macro_count, g.order, g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN, nMacN, M, N, C);
         return;
     }

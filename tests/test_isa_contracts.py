@@ -221,11 +221,11 @@ def test_hazard_checker_sees_hazards_across_branches():
 
 def test_gemm_k_loops_issue_no_other_vector_memory_instruction(tmp_path):
     text = _isa("kernels_gemm.hip", tmp_path)
-    kernels = re.findall(r"^(_ZN5spamm(?:6k_gemm|11k_gemm_half)ILi\d+ELi\d+(?:ELi\d+)?EEE\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
+    kernels = re.findall(r"^(_ZN5spamm(?:6k_gemm|10k_gemm_w64)ILi\d+ELi\d+(?:ELi\d+)?EEE\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
     # whole macro tiles by four waves: tiles 32 / 64 / 128 x ring depths 3 / 4 / 5; waves of 64 x 128 (half
     # macro tiles, whole macro tiles by eight waves): the three tiles each
-    assert len([n for n, _ in kernels if "k_gemm_half" not in n]) == 9
-    assert len([n for n, _ in kernels if "k_gemm_half" in n]) == 6
+    assert len([n for n, _ in kernels if "k_gemm_w64" not in n]) == 9
+    assert len([n for n, _ in kernels if "k_gemm_w64" in n]) == 6
     for name, body in kernels:
         mns = [mn for mn, _, _ in _instructions(body)]
         dma = [i for i, mn in enumerate(mns) if mn == "global_load_lds_dwordx4"]
