@@ -69,9 +69,13 @@ struct GateCfg {
     static constexpr uint64_t FULL = NT == 64 ? ~0ull : ((1ull << NT) - 1ull);
 };
 
-template <int MT, bool ONE>
-__global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int nMacN, float tau, int cw_arg) {
+// NTH threads per workgroup: 256, or 64 for macro tiles of 2 x 2 output tiles (tile 128), whose
+// four tiles give three of four waves nothing to do: one wave per macro tile lets four times as
+// many macro tiles be in flight on a CU, and this kernel's time is memory latency.
+template <int MT, bool ONE, int NTH = (MT == 2 ? 64 : 256)>
+__global__ __launch_bounds__(NTH) void k_gate(GateBuffers g, int nbM, int nbK, int nbN, int nMacN, float tau, int cw_arg) {
     using G = GateCfg<MT>;
+    constexpr int NW = NTH / 64;
     constexpr int NT = G::NT, NTP = G::NTP, BT = G::BT;
     extern __shared__ uint64_t smem[];
     const int words = (nbK + 63) >> 6;
@@ -147,8 +151,8 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     };
     auto build_bitmaps = [&](int w0, int cwn) {
         const int n_items = G::NQ * cwn;
-        for (int it0 = wave; it0 < n_items; it0 += 8) {
-            const int it1 = it0 + 4;
+        for (int it0 = wave; it0 < n_items; it0 += 2 * NW) {
+            const int it1 = it0 + NW;
             Item i0, i1;
             load_item(w0, it0, i0);
             if (it1 < n_items) load_item(w0, it1, i1);
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
         else return reinterpret_cast<const uint8_t *>(lmask + (size_t)wl * 8)[b];
     };
     auto transpose_words = [&](int w0, int cwn, bool record) {
-        for (int wl = wave; wl < cwn; wl += 4) {
+        for (int wl = wave; wl < cwn; wl += NW) {
             const uint64_t row = lane < NT ? lmask[(size_t)wl * NTP + lane] : 0ull;
             const uint64_t bits = transpose64(row, lane);
             const uint64_t u = __ballot(bits != 0ull), f = __ballot(bits == G::FULL);
@@ -199,7 +203,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
                 if (wave == 0 && lane < NT)
                     for (int wl = 0; wl < cwn; wl++) cnt += __builtin_popcountll(lmask[(size_t)wl * NTP + lane]);
                 const float inv_words = 1.0f / (float)cwn;     // e < 2^16, cwn <= 1024: the quotient below is exact
-                for (int e = threadIdx.x; e < NT * cwn; e += 256) {
+                for (int e = threadIdx.x; e < NT * cwn; e += NTH) {
                     const int t = (int)(((float)e + 0.5f) * inv_words), wl = e - t * cwn;
                     const int i = mi * MT + t / MT, j = mj * MT + t % MT;
                     if (i < nbM && j < nbN) g.mask[((int64_t)i * nbN + j) * words + w0 + wl] = lmask[(size_t)wl * NTP + t];
@@ -216,7 +220,7 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
                 // in ascending k rotated to the anchor: the GEMM runs a branch-free loop over the
                 // first group.
                 const int k1 = (w0 + cwn) * 64 < nbK ? (w0 + cwn) * 64 : nbK;
-                for (int k = w0 * 64 + threadIdx.x; k < k1; k += 256) {
+                for (int k = w0 * 64 + threadIdx.x; k < k1; k += NTH) {
                     const int w = k >> 6, b = k & 63;
                     const uint64_t bits = tile_bits(w - w0, b);
                     if (bits != 0ull) {
@@ -269,16 +273,16 @@ __global__ __launch_bounds__(256) void k_gate(GateBuffers g, int nbM, int nbK, i
     } else {
         // Hillis-Steele in LDS
         for (int off = 1; off <= words; off <<= 1) {
-            int addf[5], addp[5];        // words <= 1024: at most 5 per thread
+            int addf[1024 / NTH + 1], addp[1024 / NTH + 1];        // words <= 1024
             int n = 0;
-            for (int w = threadIdx.x; w <= words; w += 256) {
+            for (int w = threadIdx.x; w <= words; w += NTH) {
                 addf[n] = w >= off ? wfull[w - off] : 0;
                 addp[n] = w >= off ? wpart[w - off] : 0;
                 n++;
             }
             __syncthreads();
             n = 0;
-            for (int w = threadIdx.x; w <= words; w += 256) {
+            for (int w = threadIdx.x; w <= words; w += NTH) {
                 wfull[w] += addf[n];
                 wpart[w] += addp[n];
                 n++;
@@ -673,8 +677,8 @@ hipError_t launch_gate(const GateBuffers &g, int64_t nbM, int64_t nbK, int64_t n
     const int cw = gate_chunk_words(tile, nbK, chunk_cap);
     const bool one = cw >= (int)((nbK + 63) / 64);
 #define SPAMM_GATE(MTV)                                                                                          \
-    if (one) k_gate<MTV, true><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw);      \
-    else k_gate<MTV, false><<<n_macro, 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw)
+    if (one) k_gate<MTV, true><<<n_macro, MTV == 2 ? 64 : 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw);      \
+    else k_gate<MTV, false><<<n_macro, MTV == 2 ? 64 : 256, lds, s>>>(g, (int)nbM, (int)nbK, (int)nbN, nMacN, tau, cw)
     switch (MT) {
         case 8: SPAMM_GATE(8); break;
         case 4: SPAMM_GATE(4); break;
