@@ -410,7 +410,15 @@ static hipError_t launch_normmap(const void *X, int64_t rows, int64_t cols, int 
     // phases: tiles of a strip resident in LDS together take ~42 KiB at most (three workgroups per CU)
     switch (tile) {
         case 32: k_normmap<32, ROLE, SW, IN16, 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
-        case 64: k_normmap<64, ROLE, SW, IN16, IN16 ? 2 : 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
+        case 64:
+            // tile 64: eight waves per workgroup on fp16 input (tau-aware passes at N = 16384: 0.156 / 0.138 ->
+            // 0.152 / 0.129 ms) and, on fp32 input, for small grids (N = 8192: 0.066 / 0.058 -> 0.063 / 0.056 ms;
+            // at N = 16384 four waves are as fast or 1 % faster)
+            if (IN16 || grid <= 8192u) {
+                k_normmap<64, ROLE, SW, IN16, IN16 ? 2 : 1, 8><<<grid, 512, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip);
+                break;
+            }
+            k_normmap<64, ROLE, SW, IN16, IN16 ? 2 : 1><<<grid, 256, 0, s>>>(X, cols, cols, nbr, nbc, nstrip, (uint4 *)packed, nm, nmT, (uint4 *)packed2, nm2, rowmax, tau_skip); break;
         // tile 128: eight waves per workgroup (two 8-row groups per lane instead of four: no register
         // spills, more loads in flight) where that measured faster -- the fp32 A role (3.36 -> 3.07 ms at
         // N = 65536) and both roles on fp16 input (2.02 -> 1.85, 1.95 -> 1.90 ms) -- but not the fp32 B
