@@ -145,14 +145,16 @@ GateBuffers gate_buffers(spamm_ctx *c) {
     return g;
 }
 
-// Work unit of the gated GEMM when the caller has not fixed it: with at most one macro tile per CU
-// every workgroup runs at once and the kernel's time is one workgroup's, so halves (twice the
-// workgroups, each with half the products and three quarters of the loads) finish sooner; beyond
-// that whole macro tiles by four waves are fastest (128 flop per staged byte against 85).
+// Work unit of the gated GEMM when the caller has not fixed it: with at most half a macro tile per CU
+// halves double the workgroups that run at once (2048^3 at tile 32, 64 macro tiles: -6 %); from one
+// macro tile per CU on, whole macro tiles by four waves are as fast or faster (4096^3 dense, 256 macro
+// tiles: halves +7 %; 128 flop per staged byte against 85).  Between one and three COMPUTING macro
+// tiles per CU halves can win up to 10 % by finer rounds (270 on 256 CUs), but that count is known
+// only on the device after the gate, and the host chooses the launch.
 int gemm_shape_for(const spamm_ctx *c) {
     if (c->gemm_shape) return c->gemm_shape;
     const Shape s = shape_of(c);
-    return s.n_macro <= (int64_t)c->n_xcd * SUPER_M * SUPER_N ? GEMM_SHAPE_HALF : GEMM_SHAPE_FULL;
+    return 2 * s.n_macro <= (int64_t)c->n_xcd * SUPER_M * SUPER_N ? GEMM_SHAPE_HALF : GEMM_SHAPE_FULL;
 }
 
 int set_device(spamm_ctx *c) {
