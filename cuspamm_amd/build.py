@@ -33,6 +33,13 @@ CFLAGS = [
 ]
 
 
+# kernels_gemm.hip only.  M0 is listed as clobbered by its global->LDS loads and clang remarks on every
+# instance that M0 is reserved (it never allocates it anyway).  The ticket of the workgroups that stay is
+# drawn by one lane with a returning atomic that is asked for early and looked at late; the compiler's
+# rewrite of atomics in divergent code (one lane adds for all, then a broadcast) would wait for it at once.
+GEMM_FLAGS = ["-Wno-inline-asm", "-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]
+
+
 def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(
@@ -66,9 +73,7 @@ def build_library(verbose=False):
 
     def compile_one(pair):
         src, obj = pair
-        # kernels_gemm.hip lists M0 as clobbered by its global->LDS loads; clang remarks on every
-        # instance that M0 is a reserved register (it never allocates it anyway): silenced there
-        extra = ["-Rpass-analysis=kernel-resource-usage", "-Wno-inline-asm"] if src == "kernels_gemm.hip" else []
+        extra = ["-Rpass-analysis=kernel-resource-usage"] + GEMM_FLAGS if src == "kernels_gemm.hip" else []
         log = _run([HIPCC] + CFLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
         if extra:
             _check_no_scratch(log, src)

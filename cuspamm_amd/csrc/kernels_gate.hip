@@ -606,6 +606,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         if (lane == 0) {
             g.sched[x] = nc;
             g.sched[MAX_XCD + x] = nall;
+            g.sched[2 * MAX_XCD + x] = 0;      // ticket counter of the persistent GEMM
         }
     }
     if (threadIdx.x == 0) g.kept_total[0] = (int64_t)total;

@@ -76,14 +76,24 @@ __device__ __forceinline__ void dma_load(const unsigned char *sbase, uint32_t vo
 // workgroup barrier: after sync(t) stage t+1 is readable by all waves and no
 // wave reads stage t any more, so the loads of stage t+NBUF go into stage t's
 // buffer.  NBUF-1 stages are in flight while one is multiplied.
-template <int B, int NBUF>
+// PERSIST: the same macro tiles by workgroups that stay -- one per CU -- and take the next item of
+// their XCD's sequence from a ticket counter (what the hardware dispatcher does with one workgroup
+// per item, without ending and starting workgroups): the ticket after the current one is asked for
+// before the current item's first load, so that it has arrived when the k loops end; the next
+// item's scalar loads and prologue then run while the stores of C drain.  Nobody waits for another
+// workgroup: a ticket beyond the sequence ends the workgroup.  Every workgroup draws exactly one
+// ticket beyond the sequence, so the largest ticket (items + workgroups of the XCD - 1) is drawn
+// last, and its holder puts the counter back to zero for the next launch.  The ticket is a
+// returning atomic issued BEFORE the item's first global->LDS load: it is the oldest outstanding
+// vector-memory operation, so the hand-counted vmcnt waits below stay exact.
+template <int B, int NBUF, bool PERSIST = false>
 __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ pA,
                                               const unsigned char *__restrict__ pB,
                                               const MacroEntry *__restrict__ macro_list,
                                               const int32_t *__restrict__ macro_count,
                                               const int32_t *__restrict__ order,
-                                              const int32_t *__restrict__ sched, int P, int n_xcd, int nbM,
-                                              int nbK, int nbN, int nMacN, int64_t M, int64_t N,
+                                              const int32_t *__restrict__ sched, int32_t *__restrict__ ticket, int P,
+                                              int n_xcd, int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N,
                                               float *__restrict__ C) {
     using G = GemmCfg<B>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -98,30 +108,68 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     // write zeros; they are dispatched when CUs start to fall idle at the end
     // of the XCD's queue, so the zero-fill fills the tail of the kernel
     // instead of competing with the k loops for memory bandwidth.
-    const int xcd = blockIdx.x % n_xcd, q = blockIdx.x / n_xcd;
+    const int xcd = blockIdx.x % n_xcd;
     const int ntot = __builtin_amdgcn_readfirstlane(sched[MAX_XCD + xcd]);
-    if (q >= ntot) return;
     const int32_t *seq = order + (int64_t)xcd * P;
+    const uint32_t lds_base =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+    // persistent form: wave 0 draws the tickets and hands them to the other waves through two LDS
+    // words behind the ring, used in turn (a wave may still be reading one while the next is written)
+    int32_t *tk_word = reinterpret_cast<int32_t *>(smem + NBUF * G::STAGE_BYTES);
+    int tk_par = 0;
+    auto request = [&]() -> int {
+        int v;      // (only lane 0 of wave 0 ever looks at it; left unset elsewhere on purpose)
+        asm volatile("" : "=v"(v));
+        if (wave == 0 && lane == 0)
+            v = __hip_atomic_fetch_add(ticket + xcd, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return v;
+    };
+    auto publish = [&](int v) -> int {      // (the barrier also says: every wave has left the ring)
+        if (wave == 0 && lane == 0) tk_word[tk_par] = v;
+        __syncthreads();
+        const int r = __builtin_amdgcn_readfirstlane(tk_word[tk_par]);
+        tk_par ^= 1;
+        return r;
+    };
+    auto zero_fill = [&](int mz) {
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        int ln = lane;
+        // (workgroups that stay: keeps the lane's part of the address from being computed once for
+        // all items and held in registers through the k loops, where there are none to spare)
+        if constexpr (PERSIST) asm volatile("" : "+v"(ln));
+        const int64_t r0 = (int64_t)(mz / nMacN) * 256, c0 = (int64_t)(mz % nMacN) * 256 + ln * 4;
+        if (c0 < N)
+            for (int r = wave; r < 256 && r0 + r < M; r += 4)
+                __builtin_nontemporal_store(zero, reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0));
+    };
+    // (workgroups that stay) the holder of the largest ticket puts the counter back
+    auto last_ticket = [&](int qq) {
+        if (qq == ntot + (int)(gridDim.x / n_xcd) - 1 && threadIdx.x == 0) ticket[xcd] = 0;
+    };
+    int q, tk_next = 0;
+    if constexpr (PERSIST) q = publish(request());
+    else q = blockIdx.x / n_xcd;
+
+  // Workgroups that stay run this loop over the computing items of their XCD's sequence, then the
+  // loop at the end of the kernel over the items with nothing kept (the sequence lists them last).
+  for (;;) {
+    if (q >= ntot) {
+        if constexpr (PERSIST) last_ticket(q);
+        return;
+    }
     const int macro = __builtin_amdgcn_readfirstlane(seq[q]);
     const int mi = macro / nMacN, mj = macro % nMacN;
     const int U = __builtin_amdgcn_readfirstlane(macro_count[2 * macro]);
     const int Ufull = __builtin_amdgcn_readfirstlane(macro_count[2 * macro + 1]);
     entry_ptr ents = (entry_ptr)(uintptr_t)(macro_list + (int64_t)macro * nbK);
     const int S = U * G::NSPE, Sfull = Ufull * G::NSPE;
-    const uint32_t lds_base =
-        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
-
-    auto zero_fill = [&](int mz) {
-        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        const int64_t r0 = (int64_t)(mz / nMacN) * 256, c0 = (int64_t)(mz % nMacN) * 256 + lane * 4;
-        if (c0 < N)
-            for (int r = wave; r < 256 && r0 + r < M; r += 4)
-                __builtin_nontemporal_store(zero, reinterpret_cast<f32x4 *>(C + (r0 + r) * N + c0));
-    };
-    if (S == 0) {
-        zero_fill(macro);     // q >= nc: nothing kept in this macro tile
+    if (S == 0) {             // q >= nc: nothing kept in this macro tile
+        if constexpr (PERSIST) break;
+        zero_fill(macro);
         return;
     }
+    if constexpr (PERSIST) tk_next = request();
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -378,6 +426,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         // workgroup gives its LDS back
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     }
+    int q_next = 0;
+    if constexpr (PERSIST) q_next = publish(tk_next);
 
     // ---- epilogue: C[row, col], row-major, ld N (cuSpAMM.cu:391).  MFMA
     // 32x32 result register i of lane l is row 8*(i/4) + 4*(l/32) + i%4,
@@ -386,6 +436,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     // non-temporal stores leave the L2 to the operand panels.  (Swapping the
     // MFMA operands would give float4 stores, but each then touches 32 rows
     // with 32 bytes -- measured slower.)
+    int lane_e = lane;
+    if constexpr (PERSIST) asm volatile("" : "+v"(lane_e));     // (as in zero_fill)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const int64_t row0 = (int64_t)mi * 256 + wr * 128 + r * 32;
@@ -394,12 +446,25 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
         for (int c = 0; c < 4; c++) {
             const int64_t col0 = (int64_t)mj * 256 + wc * 128 + c * 32;
             if (col0 >= N) continue;
-            float *out = C + (row0 + 4 * (lane >> 5)) * N + col0 + (lane & 31);
+            float *out = C + (row0 + 4 * (lane_e >> 5)) * N + col0 + (lane_e & 31);
 #pragma unroll
             for (int i = 0; i < 16; i++)
                 __builtin_nontemporal_store(acc[r][c][i], &out[(int64_t)(8 * (i / 4) + (i % 4)) * N]);
         }
     }
+    if constexpr (!PERSIST) return;
+    q = q_next;
+  }
+  // (workgroups that stay) items with nothing kept: zeros, until the sequence ends
+  for (;;) {
+    tk_next = request();
+    zero_fill(__builtin_amdgcn_readfirstlane(seq[q]));
+    q = publish(tk_next);
+    if (q >= ntot) {
+        last_ticket(q);
+        return;
+    }
+  }
 }
 
 
@@ -417,6 +482,8 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 // where there is at most one macro tile per CU (chosen there); eight waves are within 1-3 %.
 constexpr int HALF_RING = 3;      // stages of the half shape's ring: 3 x 24 KiB, two workgroups per CU
 constexpr int W8_RING = 4;        // stages of the eight-wave shape's ring: 4 x 32 KiB, one workgroup per CU
+constexpr int PERSIST_RING = 4;   // stages of the persistent form's ring (k_gemm's default)
+constexpr int PERSIST_EXTRA_LDS = 16;   // the two ticket words behind the ring
 
 template <int B, int NWR>
 struct W64Cfg {
@@ -730,8 +797,12 @@ static hipError_t set_lds_attr() {
     e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_w64<B, HALF_RING, 2>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, HALF_RING * W64Cfg<B, 2>::STAGE_BYTES);
     if (e != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_w64<B, W8_RING, 4>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, W8_RING * W64Cfg<B, 4>::STAGE_BYTES);
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm_w64<B, W8_RING, 4>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, W8_RING * W64Cfg<B, 4>::STAGE_BYTES);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gemm<B, PERSIST_RING, true>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               PERSIST_RING * GemmCfg<B>::STAGE_BYTES + PERSIST_EXTRA_LDS);
 }
 
 hipError_t gemm_init() {
@@ -752,14 +823,25 @@ template <int B, int NBUF>
 static void launch_one(unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB, const GateBuffers &g,
                        int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C, hipStream_t s) {
     k_gemm<B, NBUF><<<grid, 256, NBUF * GemmCfg<B>::STAGE_BYTES, s>>>(pA, pB, g.macro_list, g.macro_count, g.order,
-                                                                     g.sched, (int)(grid / n_xcd), n_xcd, nbM, nbK, nbN,
-                                                                     nMacN, M, N, C);
+                                                                     g.sched, nullptr, (int)(grid / n_xcd), n_xcd, nbM,
+                                                                     nbK, nbN, nMacN, M, N, C);
 }
 
 template <int B>
-static void launch_tile(int nbuf, int shape, unsigned grid, int n_xcd, const unsigned char *pA, const unsigned char *pB,
-                        const GateBuffers &g, int nbM, int nbK, int nbN, int nMacN, int64_t M, int64_t N, float *C,
-                        hipStream_t s) {
+static void launch_tile(int nbuf, int shape, unsigned grid, int n_xcd, int n_cu, const unsigned char *pA,
+                        const unsigned char *pB, const GateBuffers &g, int nbM, int nbK, int nbN, int nMacN, int64_t M,
+                        int64_t N, float *C, hipStream_t s) {
+    if (shape == GEMM_SHAPE_PERSIST) {
+        // one workgroup per CU (the ring leaves room for one), an equal number on every XCD; they draw
+        // the items of their XCD's sequence from g.sched's ticket words (zero before every launch)
+        unsigned stay = (unsigned)(n_cu / n_xcd) * (unsigned)n_xcd;
+        if (stay == 0) stay = (unsigned)n_xcd;
+        if (stay > grid) stay = grid;
+        k_gemm<B, PERSIST_RING, true><<<stay, 256, PERSIST_RING * GemmCfg<B>::STAGE_BYTES + PERSIST_EXTRA_LDS, s>>>(
+            pA, pB, g.macro_list, g.macro_count, g.order, g.sched, g.sched + 2 * MAX_XCD, (int)(grid / n_xcd), n_xcd, nbM,
+            nbK, nbN, nMacN, M, N, C);
+        return;
+    }
     if (shape == GEMM_SHAPE_HALF) {
         // two workgroups per macro tile; the ring is HALF_RING stages of 24 KiB so that two workgroups fit a CU
         k_gemm_w64<B, HALF_RING, 2><<<2 * grid, 256, HALF_RING * W64Cfg<B, 2>::STAGE_BYTES, s>>>(
@@ -778,7 +860,7 @@ static void launch_tile(int nbuf, int shape, unsigned grid, int n_xcd, const uns
 }
 
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, int shape, hipStream_t s) {
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int n_cu, int ring, int shape, hipStream_t s) {
     const int MT = macro_dim(tile);
     const int nbM = (int)(M / tile), nbK = (int)(K / tile), nbN = (int)(N / tile);
     const int nMacM = (nbM + MT - 1) / MT, nMacN = (nbN + MT - 1) / MT;
@@ -788,9 +870,9 @@ hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffe
     const unsigned char *pA = (const unsigned char *)packedA;
     const unsigned char *pB = (const unsigned char *)packedB;
     switch (tile) {
-        case 32: launch_tile<32>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 64: launch_tile<64>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
-        case 128: launch_tile<128>(ring, shape, grid, n_xcd, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 32: launch_tile<32>(ring, shape, grid, n_xcd, n_cu, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 64: launch_tile<64>(ring, shape, grid, n_xcd, n_cu, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
+        case 128: launch_tile<128>(ring, shape, grid, n_xcd, n_cu, pA, pB, g, nbM, nbK, nbN, nMacN, M, N, C, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

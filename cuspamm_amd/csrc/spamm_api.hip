@@ -67,9 +67,10 @@ struct spamm_ctx : Workspace {
     hipStream_t stream = nullptr;
     int last_hip = 0;
     int n_xcd = MAX_XCD;        // XCDs the GEMM schedule is built for (from the device's CU count)
+    int n_cu = MAX_XCD * SUPER_M * SUPER_N;     // CUs of the device
     int gate_chunk_cap = 0;     // SPAMM_OPT_GATE_CHUNK_WORDS: the gate's k chunk, 0 = what LDS holds
     int gemm_ring = 4;          // SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's staging ring
-    int gemm_shape = 0;         // SPAMM_OPT_GEMM_SHAPE: 0 = chosen per call, else GEMM_SHAPE_FULL / GEMM_SHAPE_HALF
+    int gemm_shape = 0;         // SPAMM_OPT_GEMM_SHAPE: 0 = chosen per call, else one of GEMM_SHAPE_*
     uint64_t static_gen = 0;    // generation of the fixed array this context's noalloc results belong to
 
     Workspace parked;           // the workspace that is not live (see in_static)
@@ -240,6 +241,7 @@ int spamm_create(spamm_ctx **out, int device) {
     // the schedule groups workgroups by XCD (32 CUs sharing an L2): 256 CUs = 8 XCDs; a partitioned
     // device shows 128 / 64 / 32 CUs; any other CU count gets one flat sequence
     c->n_xcd = xcds_for_cu_count(prop.multiProcessorCount);
+    c->n_cu = prop.multiProcessorCount;
     int rc = set_device(c);
     if (rc == SPAMM_OK && hipStreamCreate(&c->own_stream) != hipSuccess) rc = SPAMM_EHIP;
     c->stream = c->own_stream;
@@ -305,7 +307,7 @@ int spamm_set_option(spamm_ctx *c, int option, int value) {
             c->gemm_ring = value;
             return SPAMM_OK;
         case SPAMM_OPT_GEMM_SHAPE:
-            if (value < 0 || value > 3) return SPAMM_EINVAL;
+            if (value < 0 || value > GEMM_SHAPE_PERSIST) return SPAMM_EINVAL;
             c->gemm_shape = value;
             return SPAMM_OK;
         default:
@@ -430,7 +432,7 @@ int spamm_gate(spamm_ctx *c, float tau) {
     if ((rc = ensure(c, c->macro_count, (size_t)s.n_macro * 8))) return rc;
     if ((rc = ensure(c, c->macro_work, (size_t)s.n_macro * 4))) return rc;
     if ((rc = ensure(c, c->order, (size_t)sched_rounds(c->tile, s.nbM, s.nbN) * MAX_XCD * SUPER_M * SUPER_N * 4))) return rc;
-    if ((rc = ensure(c, c->sched, 2 * MAX_XCD * 4))) return rc;
+    if ((rc = ensure(c, c->sched, SCHED_WORDS * 4))) return rc;
     if ((rc = ensure(c, c->kept_total, 16))) return rc;
     if (c->timing && !c->ev_a) HIPCHK(c, hipEventRecord(c->ev[2], c->stream));
     HIPCHK(c, launch_gate(gate_buffers(c), s.nbM, s.nbK, s.nbN, c->tile, tau, c->n_xcd, c->gate_chunk_cap, c->stream));
@@ -450,7 +452,7 @@ int spamm_gemm_gated(spamm_ctx *c, float *dC) {
     if (rc) return rc;
     if (c->timing && !c->ev_gate) HIPCHK(c, hipEventRecord(c->ev[3], c->stream));
     HIPCHK(c, launch_gemm(c->packedA.p, c->packedB.p, gate_buffers(c), c->M, c->K, c->N, c->tile, dC,
-                          c->n_xcd, c->gemm_ring, gemm_shape_for(c), c->stream));
+                          c->n_xcd, c->n_cu, c->gemm_ring, gemm_shape_for(c), c->stream));
     if (c->timing) { HIPCHK(c, hipEventRecord(c->ev[4], c->stream)); c->ev_gemm = true; }
     return SPAMM_OK;
 }
@@ -568,7 +570,7 @@ static size_t carve_static(Workspace &w, const spamm_params *p, unsigned char *b
     take(w.macro_count, n_macro * 8);
     take(w.macro_work, n_macro * 4);
     take(w.order, (size_t)sched_rounds(p->tile, (int64_t)nbM, (int64_t)nbN) * MAX_XCD * SUPER_M * SUPER_N * 4);
-    take(w.sched, 2 * MAX_XCD * 4);
+    take(w.sched, SCHED_WORDS * 4);
     take(w.kept_total, 16);
     return off;
 }

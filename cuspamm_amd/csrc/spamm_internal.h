@@ -70,7 +70,8 @@ struct GateBuffers {
     int32_t *macro_count;   // [n_macro][2]    entries in the union list, of which full (listed first)
     int32_t *macro_work;    // [n_macro]       kept products in the macro tile
     int32_t *order;         // [n_xcd * P]     macro tile of XCD x's q-th workgroup (P = rounds * 32), valid for q < sched[8 + x]
-    int32_t *sched;         // [16]            per XCD x: [x] computing items, [8 + x] all items
+    int32_t *sched;         // [24]            per XCD x: [x] computing items, [8 + x] all items, [16 + x] ticket
+                            //                 counter of the persistent GEMM (zero between launches)
     int64_t *kept_total;    // [1]  kept products
 };
 
@@ -147,9 +148,11 @@ hipError_t launch_tau_count(const float *nA, const float *nBt, int64_t nbM, int6
 
 hipError_t gemm_init();   // one-time kernel attribute set-up
 hipError_t launch_gemm(const void *packedA, const void *packedB, const GateBuffers &g, int64_t M,
-                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int ring, int shape, hipStream_t s);
-// work unit of the gated GEMM: a whole macro tile (256 x 256 of C, one workgroup per CU) or half of
-// one (128 x 256, two workgroups per CU)
-constexpr int GEMM_SHAPE_FULL = 1, GEMM_SHAPE_HALF = 2, GEMM_SHAPE_W8 = 3;
+                       int64_t K, int64_t N, int tile, float *C, int n_xcd, int n_cu, int ring, int shape, hipStream_t s);
+// work unit of the gated GEMM: a whole macro tile (256 x 256 of C, one workgroup per CU), half of
+// one (128 x 256, two workgroups per CU), a whole one by eight waves, or whole ones by workgroups
+// that stay on their CU and draw items from a ticket counter per XCD
+constexpr int GEMM_SHAPE_FULL = 1, GEMM_SHAPE_HALF = 2, GEMM_SHAPE_W8 = 3, GEMM_SHAPE_PERSIST = 4;
+constexpr int SCHED_WORDS = 3 * MAX_XCD;     // GateBuffers::sched
 
 }  // namespace spamm

@@ -102,8 +102,10 @@ SPAMM_API int spamm_destroy(spamm_ctx *ctx);
  *   SPAMM_OPT_GEMM_RING: LDS stages of the GEMM's operand ring, 3..5; 0 = default (4).
  *   SPAMM_OPT_GEMM_SHAPE: work unit of the gated GEMM: 1 = a workgroup of four waves per 256 x 256
  *     macro tile of C (one workgroup per CU), 2 = four waves per 128 x 256 half (two workgroups per
- *     CU), 3 = eight waves per macro tile; 0 = chosen per call (halves when C has at most half a
- *     macro tile per CU, else 1).  All walk the same lists in the same order: C is bit-identical.
+ *     CU), 3 = eight waves per macro tile, 4 = shape 1 by workgroups that stay on their CU and draw
+ *     macro tiles from a ticket counter per XCD; 0 = chosen per call (halves when C has at most
+ *     half a macro tile per CU, else 1).  All walk the same lists in the same order: C is
+ *     bit-identical.
  * SPAMM_EINVAL for an unknown option or a value outside its range.  The reference has no such
  * knobs: its launch shapes are compile-time constants (main.h:32-73). */
 #define SPAMM_OPT_NUM_XCD 1

@@ -113,10 +113,12 @@ def test_gate_in_small_k_chunks_gives_the_same_lists(orc, ctx, chunk_words):
         other.close()
 
 
-@pytest.mark.parametrize("shape", [2, 3])
+@pytest.mark.parametrize("shape", [2, 3, 4])
 def test_other_gemm_work_units_give_the_same_product(orc, ctx, shape):
     """The GEMM's work unit is a whole 256 x 256 macro tile by four waves (shape 1), a 128 x 256
-    half by four waves, two workgroups per CU (2), or a whole macro tile by eight waves (3).  All
+    half by four waves, two workgroups per CU (2), a whole macro tile by eight waves (3), or shape 1
+    by workgroups that stay and draw macro tiles from a ticket counter per XCD (4; every case runs
+    twice on one gate, so the counter must be back at zero after a launch).  All
     walk the macro tile's list in the same order, so C must agree bit for bit -- whole macro tiles,
     ragged edges where the lower half lies beyond the matrix, all three tile sizes, dense and empty
     regions -- and with the checker."""
@@ -146,6 +148,9 @@ def test_other_gemm_work_units_give_the_same_product(orc, ctx, shape):
             assert np.array_equal(other.get_mask(), mask)
             assert other.get_stats().kept_products == kept and 0 < kept
             assert torch.equal(got, want), (M, K, N, tile)
+            got.fill_(float("nan"))
+            other.gemm_gated(got)            # the same gate again
+            assert torch.equal(got, want), (M, K, N, tile, "second launch on one gate")
         tab = orc.decay_table("exp", 2048, 0.003)
         _check(orc, other, orc.fill_decay(384, 2048, tab, 3), orc.fill_decay(2048, 320, tab, 4), 32, 0.05)
         _check(orc, other, orc.fill_decay(640, 1024, tab, 5), orc.fill_decay(1024, 384, tab, 6), 128, 20.0)

@@ -26,8 +26,8 @@ CSRC = os.path.join(ROOT, "cuspamm_amd", "csrc")
 def _isa(src, tmp_path):
     from cuspamm_amd import build
     out = os.path.join(str(tmp_path), src.replace(".hip", ".s"))
-    cmd = [build.HIPCC] + [f for f in build.CFLAGS if f != "-Wall"] + ["-Wno-inline-asm", "-S", "--cuda-device-only",
-                                                                   os.path.join(CSRC, src), "-o", out]
+    cmd = [build.HIPCC] + [f for f in build.CFLAGS if f != "-Wall"] + build.GEMM_FLAGS + ["-S", "--cuda-device-only",
+                                                                                      os.path.join(CSRC, src), "-o", out]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert proc.returncode == 0, proc.stdout[-2000:]
     return open(out).read()
@@ -221,10 +221,12 @@ def test_hazard_checker_sees_hazards_across_branches():
 
 def test_gemm_k_loops_issue_no_other_vector_memory_instruction(tmp_path):
     text = _isa("kernels_gemm.hip", tmp_path)
-    kernels = re.findall(r"^(_ZN5spamm(?:6k_gemm|10k_gemm_w64)ILi\d+ELi\d+(?:ELi\d+)?EEE\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
-    # whole macro tiles by four waves: tiles 32 / 64 / 128 x ring depths 3 / 4 / 5; waves of 64 x 128 (half
-    # macro tiles, whole macro tiles by eight waves): the three tiles each
-    assert len([n for n, _ in kernels if "k_gemm_w64" not in n]) == 9
+    kernels = re.findall(r"^(_ZN5spamm(?:6k_gemm|10k_gemm_w64)ILi\d+ELi\d+(?:ELi\d+|ELb[01])?EEE\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
+    # whole macro tiles by four waves: tiles 32 / 64 / 128 x ring depths 3 / 4 / 5, and the three tiles by
+    # workgroups that stay (ELb1E); waves of 64 x 128 (half macro tiles, whole macro tiles by eight waves):
+    # the three tiles each
+    assert len([n for n, _ in kernels if "k_gemm_w64" not in n and "ELb0E" in n]) == 9
+    assert len([n for n, _ in kernels if "k_gemm_w64" not in n and "ELb1E" in n]) == 3
     assert len([n for n, _ in kernels if "k_gemm_w64" in n]) == 6
     for name, body in kernels:
         mns = [mn for mn, _, _ in _instructions(body)]
@@ -236,3 +238,13 @@ def test_gemm_k_loops_issue_no_other_vector_memory_instruction(tmp_path):
         # and C is stored only after the loops have drained the ring
         stores = [i for i, mn in enumerate(mns) if mn.startswith("global_store")]
         assert stores and min(i for i in stores if i > dma[0]) > dma[-1], name
+        # workgroups that stay draw their tickets with a returning atomic: it must be issued before an
+        # item's first global->LDS load (then it is older than every load the counts speak of); the
+        # stores of the previous item's C are older than the next item's loads in the same way
+        # (a third one sits in the loop over the items with nothing kept, after the last load)
+        atomics = [i for i, mn in enumerate(mns) if mn.startswith("global_atomic")]
+        if "ELb1E" in name:
+            assert len([i for i in atomics if i < dma[0]]) == 2 and len([i for i in atomics if i > dma[-1]]) == 1, name
+            assert not any(mn.startswith("scratch_") for mn in mns), name
+        else:
+            assert not atomics, name
