@@ -397,7 +397,12 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     //               N = 32768, but +1 to +3 % when most super tiles hold work (algebraic decay,
     //               30 % kept), hence the condition;
     //   DEAL_SNAKE  ranked by length, dealt in snake order (no table: any number of super tiles).
-    enum { DEAL_LPT, DEAL_BAND, DEAL_SNAKE };
+    //   DEAL_FLAT   fewer super tiles than XCDs (C of at most 7 x 32 macro tiles): whole super tiles
+    //               would leave XCDs empty -- 2048^3 at tile 32 is two of them, 64 workgroups on a
+    //               quarter of the chip -- so the macro tiles themselves are dealt, consecutive
+    //               ones in row-major order (neighbours along a row share the A panel) in equal
+    //               chunks, one per XCD; no ranking (the problem is a few microseconds long).
+    enum { DEAL_LPT, DEAL_BAND, DEAL_SNAKE, DEAL_FLAT };
     {
         int ne = 0;
         for (int sid = threadIdx.x; sid < n_super; sid += blockDim.x) ne += swork[sid] > 0;
@@ -405,9 +410,11 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     }
     __syncthreads();
     const int n_ne = s_nonempty;
-    const int deal = n_super > LPT_MAX_SUPER ? DEAL_SNAKE
+    const int deal = n_super < n_xcd ? DEAL_FLAT
+                     : n_super > LPT_MAX_SUPER ? DEAL_SNAKE
                      : (n_ne <= LPT_GREEDY_MAX ? DEAL_LPT
                         : (n_ne <= BAND_DEAL_MAX && 5 * n_ne <= 3 * n_super ? DEAL_BAND : DEAL_SNAKE));
+    const int flat_chunk = (nMacM * nMacN + n_xcd - 1) / n_xcd;      // <= P: n_super < n_xcd super tiles of 32
     // Ranking: larger key first, equal keys by smaller index; the key is the length, or in the
     // band deal just "holds work".  srank_id[rank] becomes the super tile's origin.
     //   up to RANK_SORT_MIN super tiles: rank = number of super tiles that come first, n_super^2
@@ -417,7 +424,9 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     //   >= n_super, which sort last): log^2 steps of one compare-exchange per thread instead of
     //   n_super comparisons per super tile on this one CU (150 us at 2048 super tiles).
     constexpr int RANK_SORT_MIN = 512;
-    if (n_super <= RANK_SORT_MIN) {
+    if (deal == DEAL_FLAT) {
+        // nothing to rank
+    } else if (n_super <= RANK_SORT_MIN) {
         const bool band = deal == DEAL_BAND;
         int parts = 2;
         while (parts < 32 && n_super * parts * 2 <= (int)blockDim.x) parts *= 2;
@@ -477,7 +486,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
         }
     }
     __syncthreads();
-    if (deal != DEAL_SNAKE) {
+    if (deal != DEAL_SNAKE && deal != DEAL_FLAT) {
         // lengths by rank, then the deal by one wave
         int mylen[(LPT_MAX_SUPER + 1023) / 1024], myrank[(LPT_MAX_SUPER + 1023) / 1024];
         int n = 0;
@@ -570,6 +579,7 @@ __global__ __launch_bounds__(1024) void k_order(GateBuffers g, int nMacM, int nM
     auto macro_at = [&](int x, int p) -> int {
         const int round = p / (SUPER_M * SUPER_N), slot = p % (SUPER_M * SUPER_N);
         if (p >= P) return -1;
+        if (deal == DEAL_FLAT) return (p < flat_chunk && x * flat_chunk + p < nMacM * nMacN) ? x * flat_chunk + p : -1;
         const int sr = deal != DEAL_SNAKE ? (int)sdeal[x * rounds + round] : round * n_xcd + ((round & 1) ? n_xcd - 1 - x : x);
         if (sr >= n_super) return -1;
         const int origin = srank_id[sr];

@@ -112,6 +112,22 @@ def test_macro_tile_work_lists_match_the_mask(orc, ctx, M, K, N, tile, lam, tau)
     assert sched[8:].sum() == counts.shape[0] * counts.shape[1]
 
 
+def test_small_products_are_dealt_to_every_xcd(orc, ctx):
+    """C of fewer super tiles (4 x 8 macro tiles) than the chip has XCDs: the macro tiles themselves are
+    dealt, in equal chunks of consecutive ones, so that no XCD stays empty (2048^3 at tile 32 -- the
+    reference's default experiment -- is two super tiles); a larger C goes by whole super tiles."""
+    import torch
+    for n, tile, want in ((2048, 32, [8] * 8), (1536, 64, [5, 5, 5, 5, 5, 5, 5, 1]), (1024, 128, [2] * 8)):
+        A = torch.rand((n, n), dtype=torch.float32, device="cuda")
+        ctx.multiply(A, A, tile, 0.0)
+        counts, sched = ctx.get_macro_counts()
+        assert list(sched[8:16]) == want and list(sched[:8]) == want, (n, tile, sched)
+    A = torch.rand((4096, 4096), dtype=torch.float32, device="cuda")       # 16 x 16 macro tiles = 8 super tiles
+    ctx.multiply(A, A, 64, 0.0)
+    counts, sched = ctx.get_macro_counts()
+    assert list(sched[8:16]) == [32] * 8
+
+
 def test_baseline_config1_a_equals_b(orc, ctx):
     # N=1024, A=B, exp(-0.5|i-j|), tile 32, tau=1e-4
     tab = orc.decay_table("exp", 1024, 0.5)
