@@ -5,8 +5,13 @@
 // accumulation, ascending k.  The reference gives each 32x32 output tile its
 // own block and re-fetches both operand tiles per product (16 flop/byte).
 // Here one workgroup (4 waves, 2 x 2) owns a macro tile of 256 x 256 elements
-// of C; each wave owns 128 x 128 (4 x 4 MFMA 32x32x16 accumulators = 256 fp32
-// registers per lane).  The workgroup walks the macro tile's union list of k;
+// of C; each wave owns a quarter of it, 128 x 128 elements (4 x 4 MFMA 32x32x16
+// accumulators = 256 fp32 registers per lane): the tiles in tile rows wr, wr + 2,
+// ... and tile columns wc, wc + 2, ... of the macro tile (for tiles of 128 that is
+// one tile).  Interleaved, because the tiles that keep a k at the edge of a band
+// are a corner of the macro tile: with contiguous quarters one wave would multiply
+// all of its tile pairs in such a stage and the opposite wave none.
+// The workgroup walks the macro tile's union list of k;
 // per entry it stages the needed A tiles (256 rows) and B tiles (256 columns)
 // of that k in LDS with direct global->LDS loads (a ring of NBUF stages), and every
 // wave multiplies only the (tile row, tile column) pairs whose bit is set in
@@ -279,9 +284,10 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
 
         // LDS byte offset (inside the A or B part of a stage) of this lane's
         // operand vector for MFMA block `blk` (32 of the wave's 128
-        // rows/columns) at k step kk (0 or 1) of the stage.
+        // rows/columns: block blk lies in the wave's (blk * 32 / B)-th tile
+        // row/column) at k step kk (0 or 1) of the stage.
         auto frag_off = [&](int wsel, int blk, int kk) -> int {
-            const int slot = wsel * G::SUB + (blk * 32) / B;
+            const int slot = wsel + 2 * ((blk * 32) / B);      // the wave's tile rows / columns: wsel, wsel + 2, ...
             const int ro = (blk * 32) % B;
             return slot * G::SLOT_BYTES + (((2 * kk + (lane >> 5)) * B) + ro + (lane & 31)) * 16;
         };
@@ -403,7 +409,7 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
             for (int a = 0; a < G::SUB; a++)
 #pragma unroll
                 for (int b = 0; b < G::SUB; b++) {
-                    const int bit = (wr * G::SUB + a) * G::MT + wc * G::SUB + b;
+                    const int bit = (wr + 2 * a) * G::MT + wc + 2 * b;
                     sb |= (uint32_t)((mask >> bit) & 1ull) << (a * G::SUB + b);
                 }
             load_frags(a1, b1, t, 1);
@@ -440,11 +446,11 @@ __global__ __launch_bounds__(256) void k_gemm(const unsigned char *__restrict__ 
     if constexpr (PERSIST) asm volatile("" : "+v"(lane_e));     // (as in zero_fill)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int64_t row0 = (int64_t)mi * 256 + wr * 128 + r * 32;
+        const int64_t row0 = (int64_t)mi * 256 + (wr + 2 * (r / G::RB)) * B + (r % G::RB) * 32;
         if (row0 >= M) continue;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const int64_t col0 = (int64_t)mj * 256 + wc * 128 + c * 32;
+            const int64_t col0 = (int64_t)mj * 256 + (wc + 2 * (c / G::RB)) * B + (c % G::RB) * 32;
             if (col0 >= N) continue;
             float *out = C + (row0 + 4 * (lane_e >> 5)) * N + col0 + (lane_e & 31);
 #pragma unroll
